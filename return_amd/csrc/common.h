@@ -1,0 +1,77 @@
+// Shared device helpers for the gfx950 kernels of return_amd.
+// Storage types: float, or bf16 (raw 16 bits, round-to-nearest-even on store).
+// All arithmetic is done in float.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define RA_OK 0
+#define RA_ERR_ARG 1
+#define RA_ERR_LAUNCH 2
+
+struct bf16 {
+    uint16_t x;
+};
+
+__device__ __forceinline__ float to_f(float v) { return v; }
+__device__ __forceinline__ float to_f(bf16 v) { return __uint_as_float(((uint32_t)v.x) << 16); }
+
+__device__ __forceinline__ uint16_t f2bf_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;      // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                           // round to nearest even
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_f(float f);
+template <> __device__ __forceinline__ float from_f<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16 from_f<bf16>(float f) {
+    bf16 r;
+    r.x = f2bf_bits(f);
+    return r;
+}
+
+// value rounded to the storage type and back: what a later kernel will read
+template <typename T> __device__ __forceinline__ float round_to(float f) { return to_f(from_f<T>(f)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result. scratch: >= 16 floats of LDS.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwave = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nwave; ++i) t += scratch[i];      // same order in every thread
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwave = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = scratch[0];
+    for (int i = 1; i < nwave; ++i) t = fmaxf(t, scratch[i]);
+    return t;
+}
+
+static inline int ra_launch_status() {
+    return hipGetLastError() == hipSuccess ? RA_OK : RA_ERR_LAUNCH;
+}
+
+#define RA_DTYPE_F32 0
+#define RA_DTYPE_BF16 1

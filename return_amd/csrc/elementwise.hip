@@ -1,0 +1,361 @@
+// Row-wise kernels: embedding gather, residual add + RMSNorm, per-head RMSNorm, rotary
+// rotation, cache write, the fused q/k/v preparation, SiLU-mul, residual add.
+// Formulas: rollout/fused.py:6-17 (RMSNorm), rollout/attention.py:10-25 (rotation),
+// rollout/fused.py:103-114 (SiLU-mul), rollout/cache.py:334-337 (cache write).
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= V) id = 0;          // ids are checked on the host; never read outside the table
+    const T* src = table + (size_t)id * H;
+    float* dst = out + (size_t)t * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = to_f(src[c]);
+}
+
+extern "C" int ra_embed(const void* table, const int* ids, float* out, int T, int H, int V,
+                        int dtype, void* stream) {
+    if (T <= 0) return RA_OK;
+    dim3 grid(T), block(256);
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, (hipStream_t)stream,
+                           (const float*)table, ids, out, H, V);
+    else
+        hipLaunchKernelGGL(embed_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
+                           (const bf16*)table, ids, out, H, V);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ residual add + RMSNorm
+// For output row m: r = rows ? rows[m] : m;  v = h[r] + delta[r];  out[m] = v * rsqrt(mean(v^2)+eps) * w.
+// Without a row list the sum is written back to h (the residual stream moves on);
+// with a row list h is left alone (nothing reads it afterwards).
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                   const float* __restrict__ w, float eps, T* __restrict__ out,
+                                   const int* __restrict__ rows, int H) {
+    __shared__ float scratch[16];
+    const int m = blockIdx.x;
+    const size_t r = rows ? (size_t)rows[m] : (size_t)m;
+    float* hr = h + r * H;
+    const T* dr = delta ? delta + r * H : nullptr;
+    const bool write_back = (rows == nullptr) && (delta != nullptr);
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = hr[c];
+        if (dr) v += to_f(dr[c]);
+        if (write_back) hr[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    T* o = out + (size_t)m * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = hr[c];                       // same thread wrote it above
+        if (dr && !write_back) v += to_f(dr[c]);
+        o[c] = from_f<T>(v * rstd * w[c]);
+    }
+}
+
+extern "C" int ra_add_rmsnorm(float* h, const void* delta, const float* w, float eps, void* out,
+                              const int* rows, int M, int H, int dtype, void* stream) {
+    if (M <= 0) return RA_OK;
+    dim3 grid(M), block(H >= 2048 ? 512 : 256);
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, (hipStream_t)stream, h,
+                           (const float*)delta, w, eps, (float*)out, rows, H);
+    else
+        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, grid, block, 0, (hipStream_t)stream, h,
+                           (const bf16*)delta, w, eps, (bf16*)out, rows, H);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ residual add alone
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__ delta, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) h[i] += to_f(delta[i]);
+}
+
+extern "C" int ra_residual_add(float* h, const void* delta, long long n, int dtype, void* stream) {
+    if (n <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)((n + 255) / 256));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(residual_add_kernel<float>, grid, block, 0, (hipStream_t)stream, h,
+                           (const float*)delta, (size_t)n);
+    else
+        hipLaunchKernelGGL(residual_add_kernel<bf16>, grid, block, 0, (hipStream_t)stream, h,
+                           (const bf16*)delta, (size_t)n);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ per-head RMSNorm, in place
+// x: [T, heads, D], one wave per (token, head).
+template <typename T>
+__global__ void head_rmsnorm_kernel(T* __restrict__ x, const float* __restrict__ w, float eps,
+                                    long long n_rows, int D) {
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    T* p = x + row * D;
+    float ss = 0.f;
+    for (int c = lane; c < D; c += 64) {
+        float v = to_f(p[c]);
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)D + eps);
+    for (int c = lane; c < D; c += 64) p[c] = from_f<T>(to_f(p[c]) * rstd * w[c]);
+}
+
+extern "C" int ra_head_rmsnorm(void* x, const float* w, float eps, long long n_rows, int D,
+                               int dtype, void* stream) {
+    if (n_rows <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)((n_rows + 3) / 4));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(head_rmsnorm_kernel<float>, grid, block, 0, (hipStream_t)stream,
+                           (float*)x, w, eps, n_rows, D);
+    else
+        hipLaunchKernelGGL(head_rmsnorm_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
+                           (bf16*)x, w, eps, n_rows, D);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ rotary rotation, in place
+// x: [T, heads, D]; pairs (j, j + R/2) for j < R/2; cos/sin: [max_pos, R/2] fp32.
+template <typename T>
+__global__ void rope_kernel(T* __restrict__ x, const int* __restrict__ positions,
+                            const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                            int T_tokens, int heads, int D, int R) {
+    const int half = R >> 1;
+    const long long total = (long long)T_tokens * heads * half;
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int j = (int)(i % half);
+    const long long th = i / half;               // token * heads + head
+    const int t = (int)(th / heads);
+    const int pos = positions[t];
+    const float c = cos_t[(size_t)pos * half + j], s = sin_t[(size_t)pos * half + j];
+    T* p = x + th * D;
+    const float x1 = to_f(p[j]), x2 = to_f(p[j + half]);
+    p[j] = from_f<T>(x1 * c - x2 * s);
+    p[j + half] = from_f<T>(x2 * c + x1 * s);
+}
+
+extern "C" int ra_rope(void* x, const int* positions, const float* cos_t, const float* sin_t,
+                       int T_tokens, int heads, int D, int R, int dtype, void* stream) {
+    const long long total = (long long)T_tokens * heads * (R / 2);
+    if (total <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)((total + 255) / 256));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(rope_kernel<float>, grid, block, 0, (hipStream_t)stream, (float*)x,
+                           positions, cos_t, sin_t, T_tokens, heads, D, R);
+    else
+        hipLaunchKernelGGL(rope_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (bf16*)x,
+                           positions, cos_t, sin_t, T_tokens, heads, D, R);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ split fused qkv rows into q, k, v
+template <typename T>
+__global__ void split_heads_kernel(const T* __restrict__ qkv, T* __restrict__ q, T* __restrict__ k,
+                                   T* __restrict__ v, int qw, int kw) {
+    const int t = blockIdx.x;
+    const int W = qw + 2 * kw;
+    const T* src = qkv + (size_t)t * W;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        if (c < qw) q[(size_t)t * qw + c] = src[c];
+        else if (c < qw + kw) k[(size_t)t * kw + (c - qw)] = src[c];
+        else v[(size_t)t * kw + (c - qw - kw)] = src[c];
+    }
+}
+
+extern "C" int ra_split_heads(const void* qkv, void* q, void* k, void* v, int T_tokens, int qw,
+                              int kw, int dtype, void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    dim3 grid(T_tokens), block(256);
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(split_heads_kernel<float>, grid, block, 0, (hipStream_t)stream,
+                           (const float*)qkv, (float*)q, (float*)k, (float*)v, qw, kw);
+    else
+        hipLaunchKernelGGL(split_heads_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
+                           (const bf16*)qkv, (bf16*)q, (bf16*)k, (bf16*)v, qw, kw);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ cache write
+// k, v: [T, Hkv*D] rows; pools: [rows, Hkv*D]; slot[t] = page*P + offset.
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                T* __restrict__ k_pool, T* __restrict__ v_pool,
+                                const int* __restrict__ slots, int W, long long pool_rows) {
+    const int t = blockIdx.x;
+    const long long s = slots[t];
+    if (s < 0 || s >= pool_rows) return;        // tables are built on the host; never write outside the pool
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        k_pool[s * W + c] = k[(size_t)t * W + c];
+        v_pool[s * W + c] = v[(size_t)t * W + c];
+    }
+}
+
+extern "C" int ra_kv_write(const void* k, const void* v, void* k_pool, void* v_pool,
+                           const int* slots, int T_tokens, int W, long long pool_rows, int dtype,
+                           void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    dim3 grid(T_tokens), block(256);
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, (hipStream_t)stream,
+                           (const float*)k, (const float*)v, (float*)k_pool, (float*)v_pool, slots,
+                           W, pool_rows);
+    else
+        hipLaunchKernelGGL(kv_write_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
+                           (const bf16*)k, (const bf16*)v, (bf16*)k_pool, (bf16*)v_pool, slots, W,
+                           pool_rows);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ fused q/k/v preparation
+// One wave per (token, head) over the fused projection row [q heads | k heads | v heads]:
+//   q, k heads: optional RMSNorm over D with one weight for all heads, then optional rotation
+//   by the token's position; q goes to q_out [T, Hq, D], k and v go to their cache rows.
+// D <= 512 (each lane keeps at most 4 rotary pairs and 4 pass-through values).
+#define QKV_MAX_PER_LANE 4
+template <typename T>
+__global__ void qkv_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, int D,
+                                   const float* __restrict__ wq, const float* __restrict__ wk,
+                                   float eps, const int* __restrict__ positions,
+                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                   int R, T* __restrict__ q_out, T* __restrict__ k_pool,
+                                   T* __restrict__ v_pool, const int* __restrict__ slots,
+                                   long long pool_rows, long long n_rows) {
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const int heads = Hq + 2 * Hkv;
+    const int t = (int)(row / heads);
+    const int head = (int)(row % heads);
+    const T* src = qkv + row * D;
+
+    T* dst;
+    const float* w = nullptr;
+    bool rotate = false;
+    if (head < Hq) {
+        dst = q_out + ((size_t)t * Hq + head) * D;
+        w = wq;
+        rotate = R > 0;
+    } else {
+        const int kvh = (head - Hq) % Hkv;
+        const bool is_k = head < Hq + Hkv;
+        T* pool = is_k ? k_pool : v_pool;
+        if (pool == nullptr) return;
+        const long long s = slots[t];
+        if (s < 0 || s >= pool_rows) return;
+        dst = pool + ((size_t)s * Hkv + kvh) * D;
+        if (is_k) {
+            w = wk;
+            rotate = R > 0;
+        }
+    }
+
+    const int half = R >> 1;
+    float a[QKV_MAX_PER_LANE], b[QKV_MAX_PER_LANE], p[QKV_MAX_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < QKV_MAX_PER_LANE; ++i) {
+        const int j = lane + 64 * i;
+        a[i] = b[i] = p[i] = 0.f;
+        if (j < half) {
+            a[i] = to_f(src[j]);
+            b[i] = to_f(src[j + half]);
+        }
+        const int c = R + lane + 64 * i;
+        if (c < D) p[i] = to_f(src[c]);
+        ss += a[i] * a[i] + b[i] * b[i] + p[i] * p[i];
+    }
+    float rstd = 1.f;
+    if (w != nullptr) {
+        ss = wave_sum(ss);
+        rstd = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    float cs[QKV_MAX_PER_LANE], sn[QKV_MAX_PER_LANE];
+    const int pos = rotate ? positions[t] : 0;
+#pragma unroll
+    for (int i = 0; i < QKV_MAX_PER_LANE; ++i) {
+        const int j = lane + 64 * i;
+        cs[i] = 1.f;
+        sn[i] = 0.f;
+        if (rotate && j < half) {
+            cs[i] = cos_t[(size_t)pos * half + j];
+            sn[i] = sin_t[(size_t)pos * half + j];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < QKV_MAX_PER_LANE; ++i) {
+        const int j = lane + 64 * i;
+        if (j < half) {
+            float x1 = a[i], x2 = b[i];
+            if (w != nullptr) {
+                x1 = x1 * rstd * w[j];
+                x2 = x2 * rstd * w[j + half];
+            }
+            dst[j] = from_f<T>(x1 * cs[i] - x2 * sn[i]);
+            dst[j + half] = from_f<T>(x2 * cs[i] + x1 * sn[i]);
+        }
+        const int c = R + lane + 64 * i;
+        if (c < D) {
+            float x = p[i];
+            if (w != nullptr) x = x * rstd * w[c];
+            dst[c] = from_f<T>(x);
+        }
+    }
+}
+
+extern "C" int ra_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, int D, const float* wq,
+                              const float* wk, float eps, const int* positions, const float* cos_t,
+                              const float* sin_t, int R, void* q_out, void* k_pool, void* v_pool,
+                              const int* slots, long long pool_rows, int dtype, void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    if (D > 64 * QKV_MAX_PER_LANE * 2 || R > D || (R & 1)) return RA_ERR_ARG;
+    // pairs: R/2 <= 256; pass-through: D-R <= 256
+    if ((R >> 1) > 64 * QKV_MAX_PER_LANE || (D - R) > 64 * QKV_MAX_PER_LANE) return RA_ERR_ARG;
+    const long long n_rows = (long long)T_tokens * (Hq + 2 * Hkv);
+    dim3 block(256), grid((unsigned)((n_rows + 3) / 4));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(qkv_prepare_kernel<float>, grid, block, 0, (hipStream_t)stream,
+                           (const float*)qkv, Hq, Hkv, D, wq, wk, eps, positions, cos_t, sin_t, R,
+                           (float*)q_out, (float*)k_pool, (float*)v_pool, slots, pool_rows, n_rows);
+    else
+        hipLaunchKernelGGL(qkv_prepare_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
+                           (const bf16*)qkv, Hq, Hkv, D, wq, wk, eps, positions, cos_t, sin_t, R,
+                           (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, pool_rows, n_rows);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ SiLU-mul
+// gu: [T, 2I] with the gate in the first half; out: [T, I] = silu(g) * u.
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, long long total) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long long t = i / I;
+    const int c = (int)(i % I);
+    const float g = to_f(gu[t * 2 * I + c]);
+    const float u = to_f(gu[t * 2 * I + I + c]);
+    out[i] = from_f<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int ra_silu_mul(const void* gu, void* out, int T_tokens, int I, int dtype, void* stream) {
+    const long long total = (long long)T_tokens * I;
+    if (total <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)((total + 255) / 256));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, (hipStream_t)stream,
+                           (const float*)gu, (float*)out, I, total);
+    else
+        hipLaunchKernelGGL(silu_mul_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
+                           (const bf16*)gu, (bf16*)out, I, total);
+    return ra_launch_status();
+}

@@ -1,0 +1,133 @@
+"""Engine: requests in, generated tokens out.
+
+The reference's Python entry point is ``await Engine.submit(Request(...))``
+(rollout/engine.py:341-344) with a loop that admits, prefills and decodes
+(350-409), and a response of output_ids, output_logprobs, num_tokens and
+finish_reason ("length" or "stop", rollout/engine_actor.py:66-78). This engine is
+synchronous: submit() queues a request, step() runs one scheduler step, generate()
+drives a list of prompts to the end. Token ids in, token ids out; like the
+reference's server it never tokenises.
+"""
+from __future__ import annotations
+
+import dataclasses
+import time
+from typing import Dict, List, Optional, Sequence, Union
+
+from ..config.engine import EngineConfig
+from ..sampling.params import SamplingParams, UniformStream
+from .runner import ModelRunner, StepEntry
+from .scheduler import Request, Scheduler
+
+
+@dataclasses.dataclass
+class GenerationResult:
+    """Fields of the reference's response (rollout/engine_actor.py:73-78)."""
+    output_ids: List[int]
+    output_logprobs: List[float]
+    num_tokens: int
+    finish_reason: str                      # "length" | "stop" | "error"
+    error: Optional[str] = None
+
+
+class Engine:
+    def __init__(self, model: Optional[str] = None, *, runner: Optional[ModelRunner] = None,
+                 max_token: Optional[int] = None, max_reside: Optional[int] = None,
+                 engine_config: Optional[EngineConfig] = None, **options):
+        """model: a folder with config.json and model.safetensors.
+
+        max_token (tokens the cache holds) and max_reside (most live requests) carry the
+        reference's names (rollout/server.py:90-91); other options are EngineConfig fields.
+        """
+        if runner is None:
+            ec = engine_config or EngineConfig(**options)
+            if max_token is not None:
+                ec.max_token = int(max_token)
+            if max_reside is not None:
+                ec.max_reside = int(max_reside)
+            ec.max_step_tokens = max(ec.max_step_tokens, ec.max_reside)
+            runner = ModelRunner(model, engine_config=ec)
+        self.runner = runner
+        ec = runner.engine_config
+        self.config = ec
+        self.scheduler = Scheduler(runner.cache, ec.max_reside, ec.max_step_tokens, ec.prefill_chunk,
+                                   runner.max_position)
+        self._submitted = 0
+        # running totals as in rollout/engine.py:84-125
+        self.prefill_tokens = 0
+        self.decode_tokens = 0
+        self.step_seconds = 0.0
+        self.steps = 0
+
+    # ------------------------------------------------------------------ requests
+    def submit(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
+               request_id=None) -> Request:
+        params = params or SamplingParams()
+        n = self._submitted
+        self._submitted += 1
+        r = Request(request_id if request_id is not None else n, prompt_ids, params)
+        for t in r.prompt_ids:
+            if not 0 <= t < self.runner.vocab_size:
+                raise ValueError(f"prompt token {t} outside the vocabulary of {self.runner.vocab_size}")
+        r.stream = UniformStream(self.config.seed, params.seed if params.seed is not None else n)
+        self.scheduler.add(r)
+        return r
+
+    # ------------------------------------------------------------------ one step
+    def step(self) -> List[Request]:
+        """One scheduler step; returns the requests that ended in it (finished or failed)."""
+        plan = self.scheduler.schedule()
+        ended = list(plan.failed)
+        if not plan.entries:
+            return ended
+        t0 = time.perf_counter()
+        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
+                   for e in plan.entries]
+        logits = self.runner.step(entries)
+        sampled: Dict[object, tuple] = {}
+        rows = [e.request for e in plan.entries if e.sample]
+        if rows:
+            toks, logps = self.runner.sample(
+                logits, [r.params.temperature for r in rows], [r.params.top_k for r in rows],
+                [r.params.top_p for r in rows], [r.stream.next() for r in rows])
+            for r, t, lp in zip(rows, toks, logps):
+                sampled[r.id] = (t, lp)
+        for e in plan.entries:
+            if len(e.tokens) == 1 and e.request.output:
+                self.decode_tokens += 1
+            else:
+                self.prefill_tokens += len(e.tokens)
+        ended += self.scheduler.finish_step(plan, sampled)
+        self.step_seconds += time.perf_counter() - t0
+        self.steps += 1
+        return ended
+
+    # ------------------------------------------------------------------ whole jobs
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None
+                 ) -> List[GenerationResult]:
+        """Generate for every prompt (lists of token ids); results come in the prompts' order."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling parameter sets")
+        requests = [self.submit(p, sp) for p, sp in zip(prompts, params)]
+        while self.scheduler.has_work():
+            before = (self.steps, len(self.scheduler.waiting), len(self.scheduler.running))
+            self.step()
+            if before == (self.steps, len(self.scheduler.waiting), len(self.scheduler.running)):
+                raise RuntimeError("scheduler made no progress")     # cannot happen; guards the loop
+        return [self.result_of(r) for r in requests]
+
+    @staticmethod
+    def result_of(r: Request) -> GenerationResult:
+        return GenerationResult(list(r.output), list(r.output_logprobs), len(r.output),
+                                r.finish_reason or "error", str(r.error) if r.error else None)
+
+    def stats(self) -> dict:
+        cache = self.runner.cache
+        return {"steps": self.steps, "prefill_tokens": self.prefill_tokens,
+                "decode_tokens": self.decode_tokens, "step_seconds": self.step_seconds,
+                "running": len(self.scheduler.running), "waiting": len(self.scheduler.waiting),
+                "kv_used": [g.pages.in_use() for g in cache.groups],
+                "kv_total": [g.num_pages for g in cache.groups]}

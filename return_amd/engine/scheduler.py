@@ -1,0 +1,210 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget,
+decodes, finishes and frees.
+
+What it keeps of the reference (rollout/engine.py): a queue of pending requests
+and a set of running ones (76-79); admission only while request slots are free and
+the pages the newcomer needs fit beside what running requests still need
+(_admit, 199-247); a request that can never fit fails at once with KVCapacityError
+(219-221); a request ends at max_new_tokens or on a stop sequence (49-57).
+What differs: the reference prefills all newly admitted prompts completely before
+it decodes again (358-385); here every step mixes one token of each decoding
+request with prompt portions, under max_step_tokens. And where the reference lets
+decoding requests wait for pages and fails one if none can go on (326-339), here
+pages for a request's whole life (prompt + max_new_tokens - 1 tokens) are set
+aside when it is admitted, so a running request never runs out: when pages are
+short, new requests wait in the queue, in order, until running ones finish.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+from typing import Deque, Dict, List, Optional, Sequence, Tuple
+
+from ..cache.manager import CacheManager
+from ..cache.pages import KVCapacityError
+from ..sampling.params import SamplingParams, UniformStream, ends_with_stop
+
+
+class Request:
+    """One generation request (the reference's Request, rollout/engine.py:13-62, without paragraphs)."""
+
+    def __init__(self, request_id, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None):
+        if len(prompt_ids) == 0:
+            raise ValueError(f"request {request_id!r} has an empty prompt")
+        self.id = request_id
+        self.prompt_ids = [int(t) for t in prompt_ids]
+        self.params = params or SamplingParams()
+        self.output: List[int] = []
+        self.output_logprobs: List[float] = []
+        self.num_computed = 0               # tokens of prompt + output already in the cache
+        self.status = "waiting"             # waiting | running | finished | failed
+        self.finish_reason: Optional[str] = None
+        self.error: Optional[BaseException] = None
+        self.max_new = self.params.max_new_tokens   # may be lowered to fit max_position
+        self.stream: Optional[UniformStream] = None
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.prompt_ids) + len(self.output)
+
+    def pending(self) -> List[int]:
+        """Tokens not yet in the cache: the rest of the prompt, or the last sampled token."""
+        k = self.num_computed
+        n_prompt = len(self.prompt_ids)
+        if k < n_prompt:
+            return self.prompt_ids[k:] + self.output
+        return self.output[k - n_prompt:]
+
+    @property
+    def finished(self) -> bool:
+        return self.status in ("finished", "failed")
+
+
+@dataclasses.dataclass
+class PlannedEntry:
+    request: Request
+    tokens: List[int]
+    sample: bool            # the portion reaches the request's last token: its logits are sampled
+
+
+@dataclasses.dataclass
+class StepPlan:
+    entries: List[PlannedEntry]
+    failed: List[Request]
+
+    @property
+    def n_tokens(self) -> int:
+        return sum(len(e.tokens) for e in self.entries)
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_reside: int, max_step_tokens: int,
+                 prefill_chunk: int, max_position: int):
+        if max_step_tokens < max_reside:
+            raise ValueError(
+                f"max_step_tokens {max_step_tokens} must be at least max_reside {max_reside}: "
+                f"every decoding request brings one token to every step")
+        self.cache = cache
+        self.max_reside = int(max_reside)
+        self.max_step_tokens = int(max_step_tokens)
+        self.prefill_chunk = int(prefill_chunk)
+        self.max_position = int(max_position)
+        self.max_portion = min(self.prefill_chunk, self.max_step_tokens)
+        self.waiting: Deque[Request] = collections.deque()
+        self.running: List[Request] = []
+        self._life_pages: Dict[object, List[int]] = {}     # request id -> pages of each group set aside
+
+    # ------------------------------------------------------------------ queue
+    def add(self, request: Request) -> None:
+        request.status = "waiting"
+        self.waiting.append(request)
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ------------------------------------------------------------------ accounting
+    def _unclaimed(self) -> List[int]:
+        """Free pages of each group minus what running requests may still take."""
+        free = self.cache.free_pages()
+        for r in self.running:
+            held = self.cache.held_pages(r.id)
+            for g, life in enumerate(self._life_pages[r.id]):
+                free[g] -= max(0, life - held[g])
+        return free
+
+    def _try_admit(self, r: Request) -> Optional[bool]:
+        """True: admitted. False: must wait. None: failed for good (r.error is set)."""
+        n_prompt = len(r.prompt_ids)
+        if n_prompt >= self.max_position:
+            return self._fail(r, ValueError(
+                f"prompt of {n_prompt} tokens leaves no room below max_position_embeddings "
+                f"{self.max_position}"))
+        r.max_new = min(r.params.max_new_tokens, self.max_position - n_prompt + 1)
+        life = self.cache.max_pages(n_prompt + r.max_new - 1, self.max_portion)
+        for g, need in enumerate(life):
+            if need > self.cache.groups[g].num_pages:
+                return self._fail(r, KVCapacityError(
+                    f"request needs {need} pages of cache group {g}, the pool has "
+                    f"{self.cache.groups[g].num_pages}"))
+        if len(self.running) >= self.max_reside or self.cache.free_slots() < 1:
+            return False
+        if any(need > free for need, free in zip(life, self._unclaimed())):
+            return False
+        self.cache.add_request(r.id)
+        self._life_pages[r.id] = life
+        r.status = "running"
+        self.running.append(r)
+        return True
+
+    def _fail(self, r: Request, error: BaseException):
+        r.status, r.error, r.finish_reason = "failed", error, "error"
+        return None
+
+    # ------------------------------------------------------------------ one step
+    def schedule(self) -> StepPlan:
+        """Decide the next step: one token of every decoding request, then prompt portions."""
+        budget = self.max_step_tokens
+        entries: List[PlannedEntry] = []
+        failed: List[Request] = []
+
+        def take(r: Request, limit: int):
+            nonlocal budget
+            pend = r.pending()
+            n = min(len(pend), limit, budget)
+            if n <= 0:
+                return
+            entries.append(PlannedEntry(r, pend[:n], sample=(n == len(pend))))
+            budget -= n
+
+        for r in self.running:                      # decoding requests first
+            if r.num_computed >= len(r.prompt_ids):
+                take(r, 1)
+        for r in self.running:                      # prompts under way
+            if r.num_computed < len(r.prompt_ids):
+                take(r, self.prefill_chunk)
+        while self.waiting and budget > 0:          # newcomers, in order
+            r = self.waiting[0]
+            ok = self._try_admit(r)
+            if ok is None:
+                self.waiting.popleft()
+                failed.append(r)
+                continue
+            if not ok:
+                break
+            self.waiting.popleft()
+            take(r, self.prefill_chunk)
+        return StepPlan(entries, failed)
+
+    def finish_step(self, plan: StepPlan, sampled: Dict[object, Tuple[int, float]]) -> List[Request]:
+        """Book the step: tokens are in the cache, sampled tokens join the outputs. Returns who finished."""
+        done = []
+        for e in plan.entries:
+            r = e.request
+            r.num_computed += len(e.tokens)
+            if not e.sample:
+                continue
+            tok, logp = sampled[r.id]
+            r.output.append(int(tok))
+            r.output_logprobs.append(float(logp))
+            if ends_with_stop(r.output, r.params.stop_ids):
+                r.finish_reason = "stop"
+            elif len(r.output) >= r.max_new:
+                r.finish_reason = "length"
+            if r.finish_reason:
+                r.status = "finished"
+                done.append(r)
+        for r in done:
+            self.running.remove(r)
+            self._life_pages.pop(r.id, None)
+            self.cache.free_request(r.id)
+        return done
+
+    def abort(self, r: Request, error: BaseException) -> None:
+        """Take a running or waiting request out and give back what it holds."""
+        if r in self.running:
+            self.running.remove(r)
+            self._life_pages.pop(r.id, None)
+            self.cache.free_request(r.id)
+        elif r in self.waiting:
+            self.waiting.remove(r)
+        self._fail(r, error)

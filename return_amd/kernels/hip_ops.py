@@ -1,0 +1,292 @@
+"""The kernel set of the engine: thin, checked bindings of the HIP library.
+
+Every method checks on the host that shapes, dtypes and contiguity are what the
+kernel and its grid assume, and raises before anything is launched otherwise.
+There is no other implementation behind these names: if the library cannot be
+built or loaded, constructing HipOps raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+_F32, _BF16 = 0, 1
+_c_int, _c_ll, _c_float, _c_ptr = ctypes.c_int, ctypes.c_longlong, ctypes.c_float, ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, got {dtype}")
+
+
+_LIB = None
+
+
+def load_library():
+    """The HIP library, built first if it is not there. Raises if that is impossible."""
+    global _LIB
+    if _LIB is None:
+        path = _build.ensure_built()
+        try:
+            _LIB = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load the HIP library {path}: {e}") from e
+        _declare(_LIB)
+    return _LIB
+
+
+def _declare(lib):
+    P, I, L, F = _c_ptr, _c_int, _c_ll, _c_float
+    sigs = {
+        "ra_embed": [P, P, P, I, I, I, I, P],
+        "ra_add_rmsnorm": [P, P, P, F, P, P, I, I, I, P],
+        "ra_residual_add": [P, P, L, I, P],
+        "ra_head_rmsnorm": [P, P, F, L, I, I, P],
+        "ra_rope": [P, P, P, P, I, I, I, I, I, P],
+        "ra_split_heads": [P, P, P, P, I, I, I, I, P],
+        "ra_kv_write": [P, P, P, P, P, I, I, L, I, P],
+        "ra_qkv_prepare": [P, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, L, I, P],
+        "ra_silu_mul": [P, P, I, I, I, P],
+        "ra_gemm_nt": [P, P, P, I, I, I, I, I, P],
+        "ra_attention_plain": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "ra_sample": [P, I, I, P, P, P, P, P, P],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = _c_int
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+class HipOps:
+    def __init__(self, device="cuda:0"):
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError(f"the HIP kernels run on a GPU, not on {self.device}")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to this process")
+        self.lib = load_library()
+        # float32 products must be true 32-bit wherever a library routine is used
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
+
+    # ------------------------------------------------------------------ helpers
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _check(self, status: int, name: str):
+        if status != 0:
+            why = {1: "arguments outside what the kernel takes", 2: "launch failed"}.get(status, "?")
+            raise KernelError(f"{name}: {why} (status {status})")
+
+    def _want(self, t, name, dtype=None, dims=None):
+        if t.device != self.device:
+            raise KernelError(f"{name} is on {t.device}, kernels run on {self.device}")
+        if not t.is_contiguous():
+            raise KernelError(f"{name} must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+        if dims is not None and t.dim() != dims:
+            raise KernelError(f"{name} must have {dims} dimensions, got shape {tuple(t.shape)}")
+
+    # ------------------------------------------------------------------ rows
+    def embed(self, table, ids, out):
+        self._want(table, "embedding table", dims=2)
+        self._want(ids, "token ids", torch.int32, 1)
+        self._want(out, "embedding output", torch.float32, 2)
+        T, H = out.shape
+        if ids.shape[0] != T or table.shape[1] != H:
+            raise KernelError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, out {tuple(out.shape)}")
+        self._check(self.lib.ra_embed(_ptr(table), _ptr(ids), _ptr(out), T, H, table.shape[0],
+                                      _code(table.dtype), self._stream()), "embed")
+
+    def add_rmsnorm(self, h, delta, weight, eps, out, rows=None):
+        self._want(h, "residual stream", torch.float32, 2)
+        self._want(weight, "norm weight", torch.float32, 1)
+        self._want(out, "norm output", dims=2)
+        R, H = h.shape
+        if weight.shape[0] != H or out.shape[1] != H:
+            raise KernelError(f"add_rmsnorm: h {tuple(h.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+        if delta is not None:
+            self._want(delta, "delta", out.dtype, 2)
+            if tuple(delta.shape) != (R, H):
+                raise KernelError(f"add_rmsnorm: delta {tuple(delta.shape)} does not match h {tuple(h.shape)}")
+        if rows is not None:
+            self._want(rows, "row list", torch.int32, 1)
+            M = rows.shape[0]
+        else:
+            M = R
+        if out.shape[0] != M:
+            raise KernelError(f"add_rmsnorm: out has {out.shape[0]} rows, {M} wanted")
+        self._check(self.lib.ra_add_rmsnorm(_ptr(h), _ptr(delta), _ptr(weight), float(eps), _ptr(out),
+                                            _ptr(rows), M, H, _code(out.dtype), self._stream()),
+                    "add_rmsnorm")
+
+    def residual_add(self, h, delta):
+        self._want(h, "residual stream", torch.float32)
+        self._want(delta, "delta")
+        if h.shape != delta.shape:
+            raise KernelError(f"residual_add: {tuple(h.shape)} += {tuple(delta.shape)}")
+        self._check(self.lib.ra_residual_add(_ptr(h), _ptr(delta), h.numel(), _code(delta.dtype),
+                                             self._stream()), "residual_add")
+
+    def head_rmsnorm(self, x, weight, eps):
+        self._want(x, "heads", dims=3)
+        self._want(weight, "head norm weight", torch.float32, 1)
+        if weight.shape[0] != x.shape[2]:
+            raise KernelError(f"head_rmsnorm: weight {tuple(weight.shape)} for heads {tuple(x.shape)}")
+        self._check(self.lib.ra_head_rmsnorm(_ptr(x), _ptr(weight), float(eps), x.shape[0] * x.shape[1],
+                                             x.shape[2], _code(x.dtype), self._stream()), "head_rmsnorm")
+
+    def rope(self, x, positions, cos, sin, rotary_dim):
+        self._want(x, "heads", dims=3)
+        self._want(positions, "positions", torch.int32, 1)
+        self._want(cos, "cos table", torch.float32, 2)
+        self._want(sin, "sin table", torch.float32, 2)
+        T, heads, D = x.shape
+        R = int(rotary_dim)
+        if positions.shape[0] != T or R % 2 or R > D or cos.shape[1] != R // 2 or sin.shape != cos.shape:
+            raise KernelError(f"rope: x {tuple(x.shape)}, rotary_dim {R}, tables {tuple(cos.shape)}")
+        self._check(self.lib.ra_rope(_ptr(x), _ptr(positions), _ptr(cos), _ptr(sin), T, heads, D, R,
+                                     _code(x.dtype), self._stream()), "rope")
+
+    def split_heads(self, qkv, n_q, n_kv, D, q, k, v):
+        self._want(qkv, "qkv", dims=2)
+        T = qkv.shape[0]
+        for t, name, heads in ((q, "q", n_q), (k, "k", n_kv), (v, "v", n_kv)):
+            self._want(t, name, qkv.dtype, 3)
+            if tuple(t.shape) != (T, heads, D):
+                raise KernelError(f"split_heads: {name} is {tuple(t.shape)}, wanted {(T, heads, D)}")
+        if qkv.shape[1] != (n_q + 2 * n_kv) * D:
+            raise KernelError(f"split_heads: qkv width {qkv.shape[1]} is not {(n_q + 2 * n_kv) * D}")
+        self._check(self.lib.ra_split_heads(_ptr(qkv), _ptr(q), _ptr(k), _ptr(v), T, n_q * D, n_kv * D,
+                                            _code(qkv.dtype), self._stream()), "split_heads")
+
+    def _pool_rows(self, k_pool, v_pool, n_kv, D, dtype):
+        for t, name in ((k_pool, "k pool"), (v_pool, "v pool")):
+            self._want(t, name, dtype, 4)
+            if t.shape[2] != n_kv or t.shape[3] != D:
+                raise KernelError(f"{name} {tuple(t.shape)} does not hold {n_kv} heads of {D}")
+        if k_pool.shape != v_pool.shape:
+            raise KernelError("k pool and v pool differ in shape")
+        return k_pool.shape[0] * k_pool.shape[1]
+
+    def kv_write(self, k, v, k_pool, v_pool, slot_mapping):
+        self._want(k, "k", dims=3)
+        self._want(v, "v", k.dtype, 3)
+        self._want(slot_mapping, "slot mapping", torch.int32, 1)
+        T, n_kv, D = k.shape
+        rows = self._pool_rows(k_pool, v_pool, n_kv, D, k.dtype)
+        if v.shape != k.shape or slot_mapping.shape[0] != T:
+            raise KernelError(f"kv_write: k {tuple(k.shape)}, v {tuple(v.shape)}, slots {tuple(slot_mapping.shape)}")
+        self._check(self.lib.ra_kv_write(_ptr(k), _ptr(v), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping),
+                                         T, n_kv * D, rows, _code(k.dtype), self._stream()), "kv_write")
+
+    def qkv_prepare(self, qkv, n_q, n_kv, D, w_q, w_k, eps, positions, cos, sin, rotary_dim, q_out,
+                    k_pool, v_pool, slot_mapping):
+        self._want(qkv, "qkv", dims=2)
+        self._want(q_out, "q", qkv.dtype, 3)
+        self._want(positions, "positions", torch.int32, 1)
+        self._want(slot_mapping, "slot mapping", torch.int32, 1)
+        T = qkv.shape[0]
+        R = int(rotary_dim)
+        if qkv.shape[1] != (n_q + 2 * n_kv) * D or tuple(q_out.shape) != (T, n_q, D):
+            raise KernelError(f"qkv_prepare: qkv {tuple(qkv.shape)}, q {tuple(q_out.shape)}")
+        if positions.shape[0] != T or slot_mapping.shape[0] != T:
+            raise KernelError("qkv_prepare: positions/slot mapping do not match the token count")
+        if (w_q is None) != (w_k is None):
+            raise KernelError("qkv_prepare: q and k norm weights come together")
+        if w_q is not None:
+            for w in (w_q, w_k):
+                self._want(w, "head norm weight", torch.float32, 1)
+                if w.shape[0] != D:
+                    raise KernelError(f"qkv_prepare: norm weight {tuple(w.shape)} for head size {D}")
+        if R:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if R % 2 or R > D or cos.shape[1] != R // 2 or sin.shape != cos.shape:
+                raise KernelError(f"qkv_prepare: rotary_dim {R}, tables {tuple(cos.shape)}, head size {D}")
+        if D > 512 or R // 2 > 256 or D - R > 256:
+            raise KernelError(f"qkv_prepare: head size {D} (rotary {R}) is beyond the kernel's 512")
+        rows = 0
+        if k_pool is not None:
+            rows = self._pool_rows(k_pool, v_pool, n_kv, D, qkv.dtype)
+        self._check(self.lib.ra_qkv_prepare(
+            _ptr(qkv), T, n_q, n_kv, D, _ptr(w_q), _ptr(w_k), float(eps), _ptr(positions),
+            _ptr(cos) if R else None, _ptr(sin) if R else None, R, _ptr(q_out), _ptr(k_pool),
+            _ptr(v_pool), _ptr(slot_mapping), rows, _code(qkv.dtype), self._stream()), "qkv_prepare")
+
+    def silu_mul(self, gu, out):
+        self._want(gu, "gate-up", dims=2)
+        self._want(out, "silu-mul output", gu.dtype, 2)
+        T, I = out.shape
+        if tuple(gu.shape) != (T, 2 * I):
+            raise KernelError(f"silu_mul: gate-up {tuple(gu.shape)}, out {tuple(out.shape)}")
+        self._check(self.lib.ra_silu_mul(_ptr(gu), _ptr(out), T, I, _code(gu.dtype), self._stream()),
+                    "silu_mul")
+
+    # ------------------------------------------------------------------ matrix products
+    def linear(self, x, w, out_dtype=None):
+        """y = x @ w^T, x [M, K], w [N, K]."""
+        self._want(x, "x", dims=2)
+        self._want(w, "weight", x.dtype, 2)
+        M, K = x.shape
+        N = w.shape[0]
+        if w.shape[1] != K:
+            raise KernelError(f"linear: x {tuple(x.shape)} times weight {tuple(w.shape)}^T")
+        out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and M > 0:
+            return torch.matmul(x, w.t())          # library product, as the reference's F.linear
+        y = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        self._check(self.lib.ra_gemm_nt(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(x.dtype),
+                                        _code(out_dtype), self._stream()), "gemm_nt")
+        return y
+
+    # ------------------------------------------------------------------ attention
+    def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
+        self._want(q, "q", dims=3)
+        self._want(out, "attention output", q.dtype, 3)
+        T, n_q, D = q.shape
+        g = step.groups[group]
+        n_kv = k_pool.shape[2]
+        self._pool_rows(k_pool, v_pool, n_kv, D, q.dtype)
+        if out.shape != q.shape or T != step.n_tokens:
+            raise KernelError(f"attention: q {tuple(q.shape)}, out {tuple(out.shape)}, step of {step.n_tokens}")
+        if n_q % n_kv:
+            raise KernelError(f"attention: {n_q} query heads over {n_kv} kv heads")
+        if D > 512:
+            raise KernelError(f"attention: head size {D} is beyond the kernel's 512")
+        P = k_pool.shape[1]
+        self._check(self.lib.ra_attention_plain(
+            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), _ptr(g.page_table), _ptr(g.cu_pages),
+            _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start), step.n_seqs, T, n_q, n_kv, D, P,
+            float(scale), int(window), _code(q.dtype), self._stream()), "attention_plain")
+
+    # ------------------------------------------------------------------ sampling
+    def sample(self, logits, temperature, top_k, top_p, u):
+        """Tokens and their raw log-probabilities: int32 [m, 2] (token, float bits of logprob)."""
+        self._want(logits, "logits", torch.float32, 2)
+        M, V = logits.shape
+        for t, name, dt in ((temperature, "temperature", torch.float32), (top_k, "top_k", torch.int32),
+                            (top_p, "top_p", torch.float32), (u, "uniforms", torch.float32)):
+            self._want(t, name, dt, 1)
+            if t.shape[0] != M:
+                raise KernelError(f"sample: {name} has {t.shape[0]} entries for {M} rows")
+        out = torch.empty(M, 2, dtype=torch.int32, device=self.device)
+        self._check(self.lib.ra_sample(_ptr(logits), M, V, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                       _ptr(u), _ptr(out), self._stream()), "sample")
+        return out

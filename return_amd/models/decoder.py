@@ -1,0 +1,73 @@
+"""The generic decoder: parts built from a ModelSpec, run in the order the spec gives.
+
+The reference's counterpart is the patched HF module: embed, layers in a loop,
+final norm (rollout/monkey_patch/qwen3.py:71-81), then the head on selected rows
+only (qwen3.py:145-156, rollout/model.py:286-290).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..parts.block import BLOCKS
+from ..parts.registry import part_class
+from ..parts.spec import ModelSpec
+
+
+class Decoder:
+    def __init__(self, spec: ModelSpec, weights: Dict[str, torch.Tensor], rt):
+        self.spec = spec
+        self.rt = rt
+
+        def tensors_of(ps):
+            return {role: weights[name] for role, name in ps.tensors.items()}
+
+        build = lambda cat, ps, shared=None: part_class(cat, ps.kind)(ps.params, tensors_of(ps), rt, shared)
+        self.positions = {name: build("position", ps) for name, ps in spec.positions.items()}
+        self.embedding = build("embedding", spec.embedding)
+        self.blocks = []
+        for b in spec.blocks:
+            if b.arrangement not in BLOCKS:
+                raise KeyError(f"no block arrangement {b.arrangement!r}; registered: {sorted(BLOCKS)}")
+            self.blocks.append(BLOCKS[b.arrangement](b, tensors_of, rt, self.positions))
+        self.final_norm = build("norm", spec.final_norm)
+        self.head = build("head", spec.head)
+        self.schedule = list(spec.schedule)
+        for call in self.schedule:
+            if not 0 <= call.block < len(self.blocks):
+                raise ValueError(f"run order names block {call.block}, the model has {len(self.blocks)}")
+        rt.forget_casts()
+
+    def cache_layers(self):
+        """cache layer number -> what the mixer that writes it needs (for the cache manager)."""
+        need, writers = {}, set()
+        for call in self.schedule:
+            if call.cache is None:
+                continue
+            spec = self.blocks[call.block].mixer.cache_spec()
+            if spec is None:
+                raise ValueError(f"block {call.block} keeps nothing but the run order gives it cache layer {call.cache}")
+            if call.cache in need and need[call.cache] != spec:
+                raise ValueError(f"cache layer {call.cache} is used by mixers with different needs")
+            need[call.cache] = spec
+            if call.writes_cache:
+                if call.cache in writers:
+                    raise ValueError(f"cache layer {call.cache} has two writers in the run order")
+                writers.add(call.cache)
+        missing = set(need) - writers
+        if missing:
+            raise ValueError(f"cache layers {sorted(missing)} are read but never written")
+        return need
+
+    def forward(self, step, cache):
+        """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
+        h = self.embedding.forward(step.token_ids)
+        pending = None
+        for call in self.schedule:
+            view = cache.view(call.cache) if call.cache is not None else None
+            h, pending = self.blocks[call.block].forward(h, pending, step, view, call.writes_cache)
+        if step.n_logit_rows == 0:
+            return None
+        x = self.final_norm.forward(h, pending, out_rows=step.logit_rows)
+        return self.head.forward(x)

@@ -1,0 +1,38 @@
+"""SwiGLU feed-forward: down(silu(gate(x)) * up(x)).
+
+rollout/monkey_patch/qwen3.py:20-22 with gate and up fused into one weight, gate
+rows first (qwen3.py:99-105); silu(g) * u in 32-bit: rollout/fused.py:103-114.
+"""
+from __future__ import annotations
+
+import torch
+
+from .registry import register_part
+
+
+class SwiGLU:
+    @staticmethod
+    def tensor_shapes(params):
+        H, I = params["hidden_size"], params["intermediate_size"]
+        return {"gate_proj": (I, H), "up_proj": (I, H), "down_proj": (H, I)}
+
+    @staticmethod
+    def random_init(params, role):
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.inter = int(params["intermediate_size"])
+        self.w_gate_up = torch.cat([rt.matrix(tensors["gate_proj"]), rt.matrix(tensors["up_proj"])],
+                                   dim=0).contiguous()
+        self.w_down = rt.matrix(tensors["down_proj"])
+
+    def forward(self, x, step=None):
+        ops = self.rt.ops
+        gu = ops.linear(x, self.w_gate_up)                 # [T, 2I], gate first
+        a = self.rt.empty(x.shape[0], self.inter)
+        ops.silu_mul(gu, a)
+        return ops.linear(a, self.w_down)
+
+
+register_part("feed_forward", "swiglu", SwiGLU)

@@ -1,0 +1,54 @@
+"""What every part is given at construction: device, precision, the kernels."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+_TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class Runtime:
+    """Device, compute dtype and kernel set of one engine.
+
+    dtype "bfloat16": matrices, activations and the cache are bfloat16; the residual
+    stream, norm statistics, softmax, rotation and logits are 32-bit.
+    dtype "float32": everything is 32-bit and no reduced-precision matrix mode is used.
+
+    ``ops`` is the kernel set (return_amd.kernels.hip_ops.HipOps when none is given;
+    constructing that fails loudly if the HIP library cannot be built or loaded).
+    """
+
+    def __init__(self, device="cuda:0", dtype="bfloat16", ops=None):
+        self.device = torch.device(device)
+        self.dtype_name = dtype
+        self.dtype = _TORCH_DTYPES[dtype]
+        if ops is None:
+            from ..kernels.hip_ops import HipOps
+            ops = HipOps(self.device)
+        self.ops = ops
+        self._cast: Dict[int, torch.Tensor] = {}
+
+    # ---- weight preparation -------------------------------------------------
+    def matrix(self, t: torch.Tensor) -> torch.Tensor:
+        """A matrix operand (projection, embedding table) in the compute dtype, on the device.
+
+        The same stored tensor gives the same prepared tensor (tied weights stay one copy).
+        """
+        key = (t.data_ptr(), tuple(t.shape), t.dtype)
+        hit = self._cast.get(key)
+        if hit is None:
+            hit = t.to(device=self.device, dtype=self.dtype).contiguous()
+            self._cast[key] = hit
+        return hit
+
+    def vector32(self, t: torch.Tensor) -> torch.Tensor:
+        """A small vector (norm weight) as 32-bit floats; bf16 values convert exactly."""
+        return t.to(device=self.device, dtype=torch.float32).contiguous()
+
+    def forget_casts(self) -> None:
+        self._cast.clear()
+
+    # ---- scratch ------------------------------------------------------------
+    def empty(self, *shape, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)

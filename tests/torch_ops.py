@@ -1,0 +1,154 @@
+"""A stand-in kernel set in plain torch, for tests only.
+
+It has the method names and arguments of return_amd.kernels.hip_ops.HipOps, so that
+(a) the engine's host logic (cache, step, scheduler) can be exercised on the CPU,
+and (b) every HIP kernel has a plain reference of the same call to be compared with
+on the GPU. Formulas cite the reference like the plain model does. Nothing in
+return_amd imports this file.
+"""
+from __future__ import annotations
+
+import torch
+
+
+class TorchOps:
+    def __init__(self, device="cpu"):
+        self.device = torch.device(device)
+
+    # rollout/monkey_patch/qwen3.py:73-75
+    def embed(self, table, ids, out):
+        out.copy_(table[ids.long()].float())
+
+    # rollout/fused.py:6-17 with the residual addition of qwen3.py:63,67 in front
+    def add_rmsnorm(self, h, delta, weight, eps, out, rows=None):
+        if rows is None:
+            if delta is not None:
+                h += delta.float()
+            v = h
+        else:
+            v = h[rows.long()]
+            if delta is not None:
+                v = v + delta[rows.long()].float()
+        rstd = 1.0 / torch.sqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
+        out.copy_((v * rstd * weight).to(out.dtype))
+
+    def residual_add(self, h, delta):
+        h += delta.float()
+
+    # rollout/fused.py:36-56 on a [-1, D] view
+    def head_rmsnorm(self, x, weight, eps):
+        v = x.float()
+        rstd = 1.0 / torch.sqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
+        x.copy_((v * rstd * weight).to(x.dtype))
+
+    # rollout/attention.py:10-25
+    def rope(self, x, positions, cos, sin, rotary_dim):
+        half = rotary_dim // 2
+        c = cos[positions.long()][:, None, :]
+        s = sin[positions.long()][:, None, :]
+        v = x.float()
+        x1, x2 = v[..., :half], v[..., half:rotary_dim]
+        o = torch.cat([x1 * c - x2 * s, x2 * c + x1 * s, v[..., rotary_dim:]], dim=-1)
+        x.copy_(o.to(x.dtype))
+
+    def split_heads(self, qkv, n_q, n_kv, D, q, k, v):
+        T = qkv.shape[0]
+        q.copy_(qkv[:, :n_q * D].view(T, n_q, D))
+        k.copy_(qkv[:, n_q * D:(n_q + n_kv) * D].view(T, n_kv, D))
+        v.copy_(qkv[:, (n_q + n_kv) * D:].view(T, n_kv, D))
+
+    # rollout/cache.py:334-337
+    def kv_write(self, k, v, k_pool, v_pool, slot_mapping):
+        kf = k_pool.view(-1, k_pool.shape[2], k_pool.shape[3])
+        vf = v_pool.view(-1, v_pool.shape[2], v_pool.shape[3])
+        kf[slot_mapping.long()] = k
+        vf[slot_mapping.long()] = v
+
+    def qkv_prepare(self, qkv, n_q, n_kv, D, w_q, w_k, eps, positions, cos, sin, rotary_dim, q_out,
+                    k_pool, v_pool, slot_mapping):
+        T = qkv.shape[0]
+        q = qkv[:, :n_q * D].reshape(T, n_q, D).float()
+        k = qkv[:, n_q * D:(n_q + n_kv) * D].reshape(T, n_kv, D).float()
+        v = qkv[:, (n_q + n_kv) * D:].reshape(T, n_kv, D)
+
+        def norm(x, w):
+            return x * (1.0 / torch.sqrt((x * x).sum(-1, keepdim=True) / D + eps)) * w
+
+        def rot(x):
+            half = rotary_dim // 2
+            c = cos[positions.long()][:, None, :]
+            s = sin[positions.long()][:, None, :]
+            x1, x2 = x[..., :half], x[..., half:rotary_dim]
+            return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s, x[..., rotary_dim:]], dim=-1)
+
+        if w_q is not None:
+            q, k = norm(q, w_q), norm(k, w_k)
+        if rotary_dim:
+            q, k = rot(q), rot(k)
+        q_out.copy_(q.to(q_out.dtype))
+        if k_pool is not None:
+            self.kv_write(k.to(qkv.dtype), v, k_pool, v_pool, slot_mapping)
+
+    # rollout/fused.py:103-114
+    def silu_mul(self, gu, out):
+        I = out.shape[1]
+        g, u = gu[:, :I].float(), gu[:, I:].float()
+        out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+
+    # rollout/monkey_patch/qwen3.py:21 (F.linear)
+    def linear(self, x, w, out_dtype=None):
+        return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
+
+    # rollout/attention.py:126-139 over the tables of rollout/cache.py:282-328,
+    # gathered as opd/test_parallel.py:14-42 does
+    def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
+        g = step.groups[group]
+        P = k_pool.shape[1]
+        n_q, n_kv = q.shape[1], k_pool.shape[2]
+        cu_q, cu_p = step.cu_q.tolist(), g.cu_pages.tolist()
+        q_start, kv_start = step.q_start.tolist(), g.kv_start.tolist()
+        table = g.page_table.long()
+        for s in range(step.n_seqs):
+            a, b = cu_q[s], cu_q[s + 1]
+            pages = table[cu_p[s]:cu_p[s + 1]]
+            end = q_start[s] + (b - a)                      # keys held after this step
+            k = k_pool[pages].reshape(-1, n_kv, k_pool.shape[3])[:end - kv_start[s]].float()
+            v = v_pool[pages].reshape(-1, n_kv, v_pool.shape[3])[:end - kv_start[s]].float()
+            k_pos = torch.arange(kv_start[s], end, device=q.device)
+            q_pos = torch.arange(q_start[s], end, device=q.device)
+            kk = k.repeat_interleave(n_q // n_kv, dim=1)
+            vv = v.repeat_interleave(n_q // n_kv, dim=1)
+            score = torch.einsum("qhd,khd->hqk", q[a:b].float(), kk) * scale
+            hide = k_pos[None, :] > q_pos[:, None]
+            if window:
+                hide = hide | (k_pos[None, :] <= q_pos[:, None] - window)
+            score = score.masked_fill(hide[None], float("-inf"))
+            out[a:b] = torch.einsum("hqk,khd->qhd", score.softmax(-1), vv).to(out.dtype)
+
+    # rollout/model.py:15-61 with the draw made by inverse CDF in vocabulary order
+    def sample(self, logits, temperature, top_k, top_p, u):
+        M, V = logits.shape
+        res = torch.empty(M, 2, dtype=torch.int32, device=logits.device)
+        for r in range(M):
+            row = logits[r].double()
+            t = float(temperature[r])
+            if t <= 0:
+                tok = int(row.argmax())
+            else:
+                x = row / t
+                vals, idx = torch.sort(x, descending=True, stable=True)
+                k = int(top_k[r]) if int(top_k[r]) > 0 else V
+                vals = vals.masked_fill(torch.arange(V, device=x.device) >= k, float("-inf"))
+                cum = vals.softmax(-1).cumsum(-1)
+                remove = cum > float(top_p[r])
+                remove[1:] = remove[:-1].clone()
+                remove[0] = False
+                vals = vals.masked_fill(remove, float("-inf"))
+                p = torch.zeros(V, dtype=torch.float64, device=x.device)
+                p[idx] = vals.softmax(-1)
+                c = p.cumsum(-1)
+                tok = int((c > float(u[r]) * float(c[-1])).nonzero()[0]) if float(u[r]) < 1 else V - 1
+            lp = float(row.log_softmax(-1)[tok])
+            res[r, 0] = tok
+            res[r, 1] = torch.tensor(lp, dtype=torch.float32).view(torch.int32)
+        return res
