@@ -1,0 +1,296 @@
+"""Each HIP kernel alone against its plain torch reference (tests/torch_ops.py), at sizes
+other than the engine configurations': widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd head counts."""
+import types
+
+import pytest
+import torch
+
+from tests.torch_ops import TorchOps
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from return_amd.kernels.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchOps(DEV)
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(331, 120, 7), (1000, 4096, 3)])
+def test_embed(ops, ref, dtype, V, H, T):
+    table = rnd(V, H, dtype=dtype)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32, device=DEV)
+    a = torch.empty(T, H, dtype=torch.float32, device=DEV)
+    b = torch.empty_like(a)
+    ops.embed(table, ids, a)
+    ref.embed(table, ids, b)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("R,H", [(5, 120), (33, 1000), (3, 5120)])
+@pytest.mark.parametrize("mode", ["plain", "delta", "rows", "delta_rows"])
+def test_add_rmsnorm(ops, ref, dtype, R, H, mode):
+    h = rnd(R, H, seed=1, scale=3.0)
+    delta = rnd(R, H, dtype=dtype, seed=2) if "delta" in mode else None
+    rows = torch.tensor([R - 1, 0, R // 2], dtype=torch.int32, device=DEV) if "rows" in mode else None
+    w = 1.0 + 0.1 * rnd(H, seed=3)
+    M = R if rows is None else 3
+    ha, hb = h.clone(), h.clone()
+    a = torch.empty(M, H, dtype=dtype, device=DEV)
+    b = torch.empty_like(a)
+    ops.add_rmsnorm(ha, delta, w, 1e-5, a, rows)
+    ref.add_rmsnorm(hb, delta, w, 1e-5, b, rows)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    torch.testing.assert_close(ha, hb, atol=1e-6, rtol=1e-6)
+    if rows is not None:
+        assert torch.equal(ha, h)          # with a row list the residual stream is left alone
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_mean_square_is_one(ops, dtype):
+    """With weight 1 the output row has mean square 1/(1 + eps/ms): the norm divides by the RMS."""
+    h = rnd(4, 777, seed=5, scale=7.0)
+    w = torch.ones(777, device=DEV)
+    out = torch.empty(4, 777, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h, None, w, 1e-6, out, None)
+    ms = (out.float() ** 2).mean(-1)
+    torch.testing.assert_close(ms, torch.ones_like(ms), atol=1e-2 if dtype == torch.bfloat16 else 1e-5, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D", [16, 48, 80, 128, 256])
+def test_head_rmsnorm_and_rope(ops, ref, dtype, D):
+    T, heads = 9, 5
+    x = rnd(T, heads, D, dtype=dtype, seed=D)
+    w = 1.0 + 0.1 * rnd(D, seed=7)
+    a, b = x.clone(), x.clone()
+    ops.head_rmsnorm(a, w, 1e-6)
+    ref.head_rmsnorm(b, w, 1e-6)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    for R in (D, D // 2 if (D // 2) % 2 == 0 else D):
+        pos = torch.tensor([0, 1, 2, 100, 299, 7, 8, 9, 10], dtype=torch.int32, device=DEV)
+        ang = torch.outer(torch.arange(300, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(0, R // 2).float() / (R // 2))))
+        cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+        a, b = x.clone(), x.clone()
+        ops.rope(a, pos, cos, sin, R)
+        ref.rope(b, pos, cos, sin, R)
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+        assert torch.equal(a[0], x[0])     # position 0 is the identity
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,R,norm", [(4, 2, 16, 16, True), (6, 1, 32, 32, True), (5, 5, 48, 48, True),
+                                           (3, 1, 80, 32, False), (8, 2, 128, 128, True),
+                                           (2, 2, 256, 64, True), (1, 1, 512, 512, True)])
+def test_qkv_prepare(ops, ref, dtype, Hq, Hkv, D, R, norm):
+    T, P, pages = 11, 8, 6
+    qkv = rnd(T, (Hq + 2 * Hkv) * D, dtype=dtype, seed=11)
+    wq = 1.0 + 0.1 * rnd(D, seed=12) if norm else None
+    wk = 1.0 + 0.1 * rnd(D, seed=13) if norm else None
+    pos = torch.arange(20, 20 + T, dtype=torch.int32, device=DEV)
+    ang = torch.outer(torch.arange(64, dtype=torch.float32), 1.0 / (1e6 ** (torch.arange(0, R // 2).float() / (R // 2))))
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    slots = torch.randperm(P * pages)[:T].to(torch.int32).to(DEV)
+    outs = []
+    for o in (ops, ref):
+        q = torch.zeros(T, Hq, D, dtype=dtype, device=DEV)
+        kp = torch.zeros(pages, P, Hkv, D, dtype=dtype, device=DEV)
+        vp = torch.zeros_like(kp)
+        o.qkv_prepare(qkv, Hq, Hkv, D, wq, wk, 1e-6, pos, cos, sin, R, q, kp, vp, slots)
+        outs.append((q, kp, vp))
+    for a, b in zip(*outs):
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    # without pools nothing is written and q is the same
+    q2 = torch.zeros(T, Hq, D, dtype=dtype, device=DEV)
+    ops.qkv_prepare(qkv, Hq, Hkv, D, wq, wk, 1e-6, pos, cos, sin, R, q2, None, None, slots)
+    assert torch.equal(q2, outs[0][0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_split_and_kv_write(ops, ref, dtype):
+    T, Hq, Hkv, D, P, pages = 6, 3, 2, 48, 4, 5
+    qkv = rnd(T, (Hq + 2 * Hkv) * D, dtype=dtype, seed=21)
+    slots = torch.randperm(P * pages)[:T].to(torch.int32).to(DEV)
+    res = []
+    for o in (ops, ref):
+        q = torch.empty(T, Hq, D, dtype=dtype, device=DEV)
+        k = torch.empty(T, Hkv, D, dtype=dtype, device=DEV)
+        v = torch.empty_like(k)
+        o.split_heads(qkv, Hq, Hkv, D, q, k, v)
+        kp = torch.zeros(pages, P, Hkv, D, dtype=dtype, device=DEV)
+        vp = torch.zeros_like(kp)
+        o.kv_write(k, v, kp, vp, slots)
+        res.append((q, k, v, kp, vp))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(3, 200), (17, 1111)])
+def test_silu_mul(ops, ref, dtype, T, I):
+    gu = rnd(T, 2 * I, dtype=dtype, seed=31, scale=3.0)
+    a = torch.empty(T, I, dtype=dtype, device=DEV)
+    b = torch.empty_like(a)
+    ops.silu_mul(gu, a)
+    ref.silu_mul(gu, b)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(1, 331, 120), (7, 100, 77), (64, 64, 64), (65, 129, 250), (200, 48, 1000)])
+def test_linear(ops, dtype, out_dtype, M, N, K):
+    x = rnd(M, K, dtype=dtype, seed=41)
+    w = rnd(N, K, dtype=dtype, seed=42, scale=0.1)
+    y = ops.linear(x, w, out_dtype=out_dtype)
+    want = x.double() @ w.double().t()
+    assert y.dtype == out_dtype and tuple(y.shape) == (M, N)
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(y.double(), want, atol=2e-5 * K ** 0.5, rtol=1e-5)
+    else:
+        torch.testing.assert_close(y.double(), want, atol=3e-2, rtol=2e-2)
+
+
+def test_linear_fp32_is_true_fp32(ops):
+    """A product that bf16 or tf32 inputs would get wrong: 1 + 2^-20 squared sums."""
+    K = 512
+    x = torch.full((4, K), 1.0 + 2.0 ** -20, device=DEV)
+    w = torch.full((8, K), 1.0 + 2.0 ** -20, device=DEV)
+    y = ops.linear(x, w)
+    want = K * (1.0 + 2.0 ** -20) ** 2
+    assert abs(float(y[0, 0]) - want) < 1e-3 * 2.0 ** -10 * K
+
+
+def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
+    """A StepBatch-like object for the attention ops from host lists."""
+    n = len(q_lens)
+    cu_q = [0]
+    for q in q_lens:
+        cu_q.append(cu_q[-1] + q)
+    cu_p = [0]
+    for p in pages_of:
+        cu_p.append(cu_p[-1] + len(p))
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    g = types.SimpleNamespace(page_table=i32([p for ps in pages_of for p in ps]), cu_pages=i32(cu_p),
+                              kv_start=i32(kv_starts or [0] * n), slot_mapping=None,
+                              n_pages=[len(p) for p in pages_of], max_pages=max(len(p) for p in pages_of))
+    return types.SimpleNamespace(n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
+                                 seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
+                                 q_lens=list(q_lens), q_starts=list(q_starts),
+                                 all_decode=all(q == 1 for q in q_lens), max_q_len=max(q_lens),
+                                 max_seq_len=max(a + b for a, b in zip(q_starts, q_lens)))
+
+
+ATTN_CASES = [
+    # Hq, Hkv, D, P, [(q_len, q_start)], window
+    (4, 2, 16, 16, [(5, 0), (17, 0), (33, 0)], 0),
+    (6, 1, 32, 32, [(1, 99), (24, 8), (1, 0), (2, 62)], 0),
+    (5, 5, 48, 16, [(40, 3), (1, 200)], 0),
+    (8, 2, 128, 16, [(1, 500), (1, 17), (1, 0), (1, 255)], 0),
+    (8, 2, 128, 64, [(130, 0), (70, 190)], 0),
+    (4, 4, 80, 8, [(30, 10), (1, 77)], 12),
+    (3, 1, 64, 16, [(64, 64), (1, 128)], 33),
+    (2, 1, 256, 16, [(19, 30)], 0),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,P,segs,window", ATTN_CASES)
+def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
+    q_lens = [s[0] for s in segs]
+    q_starts = [s[1] for s in segs]
+    need = [-(-(a + b) // P) for a, b in segs]
+    total_pages = sum(need) + 3
+    perm = torch.randperm(total_pages, generator=torch.Generator().manual_seed(5)).tolist()
+    pages_of = []
+    for k in need:
+        pages_of.append([perm.pop() for _ in range(k)])
+    step = _step(q_lens, q_starts, P, pages_of)
+    kp = rnd(total_pages, P, Hkv, D, dtype=dtype, seed=51)
+    vp = rnd(total_pages, P, Hkv, D, dtype=dtype, seed=52)
+    q = rnd(sum(q_lens), Hq, D, dtype=dtype, seed=53)
+    a = torch.zeros_like(q)
+    b = torch.zeros_like(q)
+    ops.attention(q, a, kp, vp, step, 0, D ** -0.5, window)
+    ref.attention(q, b, kp, vp, step, 0, D ** -0.5, window)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_far_key_stands_out(ops, dtype):
+    """One key far back among hundreds is made to dominate: the output must be its value."""
+    Hq, Hkv, D, P, L = 4, 2, 64, 16, 700
+    pages = list(range(-(-L // P)))
+    step = _step([1], [L - 1], P, [pages])
+    kp = rnd(len(pages), P, Hkv, D, dtype=dtype, seed=61, scale=0.1)
+    vp = rnd(len(pages), P, Hkv, D, dtype=dtype, seed=62)
+    q = rnd(1, Hq, D, dtype=dtype, seed=63, scale=0.1)
+    far = 37
+    kp.view(-1, Hkv, D)[far] = (q.view(Hq, D)[::2] * 400).to(dtype)      # kv head h gets query head 2h, scaled up
+    out = torch.zeros_like(q)
+    ops.attention(q, out, kp, vp, step, 0, 1.0, 0)
+    want = vp.view(-1, Hkv, D)[far].float()
+    torch.testing.assert_close(out[0, ::2].float(), want, atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("V", [331, 5000])
+def test_sample_greedy_and_logprob(ops, V):
+    logits = rnd(6, V, seed=71, scale=3.0)
+    z = torch.zeros(6, device=DEV)
+    out = ops.sample(logits, z, torch.zeros(6, dtype=torch.int32, device=DEV), torch.ones(6, device=DEV), z)
+    tok = out[:, 0].long()
+    assert torch.equal(tok, logits.argmax(-1))
+    lp = out[:, 1].contiguous().view(torch.float32)
+    want = logits.double().log_softmax(-1).gather(1, tok[:, None])[:, 0]
+    torch.testing.assert_close(lp.double(), want, atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("V", [97, 1000])
+def test_sample_matches_plain_draw(ops, ref, V):
+    M = 64
+    logits = rnd(M, V, seed=72, scale=2.0)
+    g = torch.Generator().manual_seed(9)
+    u = torch.rand(M, generator=g).to(DEV)
+    temp = torch.tensor([0.7, 1.0, 1.3, 0.0] * (M // 4), device=DEV)
+    top_k = torch.tensor([0, 5, 0, 3, 50, 0, 1, 0] * (M // 8), dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.3, 0.0, 1.0, 0.95] * (M // 8), device=DEV)
+    a = ops.sample(logits, temp, top_k, top_p, u)
+    b = ref.sample(logits, temp, top_k, top_p, u)
+    same = (a[:, 0] == b[:, 0]).float().mean().item()
+    assert same == 1.0, (a[:, 0].tolist(), b[:, 0].tolist())
+    torch.testing.assert_close(a[:, 1].contiguous().view(torch.float32), b[:, 1].contiguous().view(torch.float32),
+                               atol=1e-4, rtol=1e-5)
+
+
+def test_sample_distribution(ops):
+    """Plain temperature sampling draws from softmax(logits / T): chi-square on a tiny vocabulary."""
+    V, N = 7, 20000
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5, 1.5, -2.0]], device=DEV).repeat(N, 1)
+    u = torch.rand(N, generator=torch.Generator().manual_seed(1)).to(DEV)
+    temp = torch.full((N,), 0.8, device=DEV)
+    out = ops.sample(logits, temp, torch.zeros(N, dtype=torch.int32, device=DEV), torch.ones(N, device=DEV), u)
+    counts = torch.bincount(out[:, 0].long().cpu(), minlength=V).double()
+    p = (logits[0].double().cpu() / 0.8).softmax(-1)
+    chi2 = float(((counts - N * p) ** 2 / (N * p)).sum())
+    assert chi2 < 30.0, (chi2, counts.tolist())

@@ -1,0 +1,100 @@
+"""Replay on the GPU: the same requests whole, with a decoded tail, in portions of changing
+size and mixed with page reuse, in 32-bit and in bfloat16, against the plain implementation."""
+import pytest
+import torch
+
+from tests import trace_tools as tt
+from tests.conftest import TINY_A, TINY_B, TINY_C
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 150, "g": 1, "h": 47}
+TOL = {"float32": dict(atol=2e-4, rtol=2e-4), "bfloat16": dict(atol=6e-2, rtol=5e-2)}
+
+
+def requests_for(vocab, max_pos):
+    return {rid: tt.random_tokens(vocab, min(n, max_pos), seed=ord(rid)) for rid, n in LENGTHS.items()}
+
+
+def oracle(folder, requests):
+    cfg, w = plain.read_folder(folder)
+    return {rid: plain.logits(cfg, w, toks) for rid, toks in requests.items()}
+
+
+def make_runner(folder, dtype, max_tokens, page=16):
+    from return_amd.config import EngineConfig
+    from return_amd.engine import ModelRunner
+    ec = EngineConfig(dtype=dtype, page_size=page, max_token=max_tokens, max_reside=4,
+                      max_step_tokens=max(max_tokens, 4), prefill_chunk=max_tokens)
+    return ModelRunner(folder, engine_config=ec)
+
+
+def compare(got, want, requests, dtype):
+    worst = 0.0
+    for rid, toks in requests.items():
+        for p in range(len(toks)):
+            assert (rid, p) in got, f"no logits for request {rid} position {p}"
+            a, b = got[(rid, p)], want[rid][p]
+            err = (a - b).abs().max().item()
+            worst = max(worst, err)
+            try:
+                torch.testing.assert_close(a, b, **TOL[dtype])
+            except AssertionError as e:
+                raise AssertionError(f"request {rid} position {p} (first wrong place): {e}") from None
+            if dtype == "float32":
+                assert int(a.argmax()) == int(b.argmax()), f"request {rid} position {p}: argmax differs"
+    return worst
+
+
+@pytest.fixture(scope="module", params=["a", "b", "c"])
+def model(request, folder_a, folder_b, folder_c):
+    folder = {"a": folder_a, "b": folder_b, "c": folder_c}[request.param]
+    raw = {"a": TINY_A, "b": TINY_B, "c": TINY_C}[request.param]
+    reqs = requests_for(raw["vocab_size"], raw["max_position_embeddings"])
+    return folder, raw, reqs, oracle(folder, reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail_decoded", "portions", "mixed"])
+def test_replay_matches_plain(model, dtype, cut):
+    folder, raw, reqs, want = model
+    steps = {"whole": tt.whole, "tail_decoded": tt.tail_decoded, "portions": tt.portions,
+             "mixed": tt.mixed}[cut](reqs)
+    # the pool holds exactly the trace's peak, so pages of ended requests are used again
+    runner = make_runner(folder, dtype, tt.peak_tokens(steps))
+    got = tt.run_in_process(runner, steps)
+    compare(got, want, reqs, dtype)
+    assert not runner.cache.live
+    assert all(g.pages.in_use() == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("page", [8, 32, 64])
+def test_other_page_sizes(folder_b, page):
+    reqs = requests_for(TINY_B["vocab_size"], TINY_B["max_position_embeddings"])
+    want = oracle(folder_b, reqs)
+    steps = tt.mixed(reqs, seed=page)
+    runner = make_runner(folder_b, "float32", tt.peak_tokens(steps, page) + page * 2, page)
+    compare(tt.run_in_process(runner, steps), want, reqs, "float32")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folder_a, tmp_path, dtype):
+    """The program itself, as a child process: stdin steps, done lines, .f32 files."""
+    reqs = requests_for(TINY_A["vocab_size"], TINY_A["max_position_embeddings"])
+    reqs = {k: reqs[k] for k in ("a", "b", "c", "d", "e")}
+    want = oracle(folder_a, reqs)
+    steps = tt.mixed(reqs, seed=3)
+    got = tt.run_program(folder_a, dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps),
+                         TINY_A["vocab_size"])
+    compare(got, want, reqs, dtype)
+
+
+def test_long_decoding(folder_b):
+    """300 tokens one by one after a short prompt, in 32-bit."""
+    toks = tt.random_tokens(TINY_B["vocab_size"], 320, seed=77)
+    reqs = {"long": toks}
+    want = oracle(folder_b, reqs)
+    steps = tt.tail_decoded(reqs, tail=300)
+    runner = make_runner(folder_b, "float32", 320)
+    compare(tt.run_in_process(runner, steps), want, reqs, "float32")
