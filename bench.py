@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, Qwen3-8B shape, random weights.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the whole batch through the engine's own step function and
+sampler (greedy), as generation runs it. Prints ONE JSON line. For --gpus > 1 it says that
+this engine runs on one GPU and exits with 2.
+
+What the reference's benches measure (definitions only, no numbers are published):
+decode tok/s = bs*steps/wall after warm-up (rollout/utils/bench_sym.py:24-62), prefill
+tok/s = ctx/mean(dt) (rollout/utils/bench_prefill.py:22-49).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+# BASELINE.json configs[2]: Qwen3-8B shape
+QWEN3_8B = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936, hidden_size=4096,
+    num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+    intermediate_size=12288, max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1e6,
+    tie_word_embeddings=False)
+FULL_LAYERS = 36
+CONTEXT = 2048          # every request's prefix when decoding starts
+MAX_CONTEXT = 8192      # the cache holds this many tokens per request
+PAGE = 16
+PREFILL_TOKENS = 2048
+
+
+def build_runner(layers, dtype, max_reside, seed=0):
+    import torch
+    import return_amd.models  # noqa: F401
+    from return_amd.config import EngineConfig, Qwen3Config
+    from return_amd.engine import ModelRunner
+    from return_amd.config import lookup_architecture
+    from return_amd.weights import random_weights
+
+    raw = dict(QWEN3_8B, num_hidden_layers=layers)
+    cfg = Qwen3Config.from_dict(raw)
+    _, build_spec = lookup_architecture(cfg.architecture)
+    weights = random_weights(build_spec(cfg), seed=seed, std=0.02, dtype=dtype, device="cuda:0",
+                             generator_device="cuda:0")
+    ec = EngineConfig(dtype=dtype, page_size=PAGE, max_token=max_reside * MAX_CONTEXT,
+                      max_reside=max_reside, max_step_tokens=max(PREFILL_TOKENS, max_reside),
+                      prefill_chunk=PREFILL_TOKENS)
+    runner = ModelRunner(config=cfg, weights=weights, engine_config=ec)
+    del weights
+    torch.cuda.empty_cache()
+    return cfg, runner
+
+
+def weight_bytes(cfg, elt):
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    per_layer = ((cfg.q_width + 2 * cfg.kv_width) * H + H * cfg.q_width + 3 * H * I) * elt + 2 * H * 4 \
+        + 2 * cfg.head_dim * 4
+    return cfg.num_hidden_layers * per_layer + V * H * elt + H * 4
+
+
+def kv_bytes_per_token(cfg, elt):
+    return 2 * cfg.kv_width * elt * cfg.num_hidden_layers
+
+
+def prefill_flops(cfg, T):
+    H, I = cfg.hidden_size, cfg.intermediate_size
+    linear = ((cfg.q_width + 2 * cfg.kv_width) * H + H * cfg.q_width + 3 * H * I) * cfg.num_hidden_layers
+    attn = cfg.num_hidden_layers * 2 * T * T * cfg.num_attention_heads * cfg.head_dim   # causal QK^T + PV
+    return 2 * T * linear + attn + 2 * cfg.vocab_size * H
+
+
+def seat_requests(runner, batch, context, seed=1):
+    """Live requests that already hold ``context`` tokens: pages are taken through the cache
+    manager and filled with random keys and values (their content does not change the work)."""
+    import torch
+    ids = [f"r{i}" for i in range(batch)]
+    for rid in ids:
+        runner.add_request(rid)
+        runner.cache.begin_step([(rid, context)])
+        runner.cache.end_step()
+    g = torch.Generator(device="cuda:0").manual_seed(seed)
+    for grp in runner.cache.groups:
+        grp.pool.normal_(0.0, 0.5, generator=g)
+    return ids
+
+
+def decode_steps(runner, ids, steps, warmup, vocab):
+    """warmup untimed steps, then exactly ``steps`` timed; returns seconds."""
+    import torch
+    from return_amd.engine import StepEntry
+    n = len(ids)
+    toks = [(7 * i + 3) % vocab for i in range(n)]
+    zeros, ones = [0.0] * n, [1.0] * n
+
+    def one():
+        nonlocal toks
+        logits = runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)])
+        toks, _ = runner.sample(logits, zeros, [0] * n, ones, zeros)
+
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def release(runner, ids):
+    for rid in ids:
+        runner.free_request(rid)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible")
+        return 1
+    elt = 2 if args.dtype == "bfloat16" else 4
+    cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch))
+    V = cfg.vocab_size
+
+    # ---- headline: decode at the given batch
+    ids = seat_requests(runner, args.batch, CONTEXT)
+    secs = decode_steps(runner, ids, args.steps, args.warmup, V)
+    release(runner, ids)
+    ms_step = secs / args.steps * 1e3
+    value = args.batch * args.steps / secs
+    mean_ctx = CONTEXT + args.warmup + (args.steps + 1) / 2.0
+    step_bytes = weight_bytes(cfg, elt) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elt)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+
+    points, prefill = {}, None
+    if not args.no_points:
+        for b in (1, 64):
+            ids = seat_requests(runner, b, CONTEXT)
+            k = max(8, min(args.steps, 32))
+            s = decode_steps(runner, ids, k, min(args.warmup, 4), V)
+            release(runner, ids)
+            points[f"decode_b{b}"] = round(b * k / s, 1)
+        # ---- prefill of one 2,048-token prompt, logits at the last place
+        from return_amd.engine import StepEntry
+        prompt = [(13 * i + 5) % V for i in range(PREFILL_TOKENS)]
+        times = []
+        for it in range(4):
+            runner.add_request("p")
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = runner.step([StepEntry("p", prompt, [PREFILL_TOKENS - 1])])
+            out.sum().item()
+            times.append(time.perf_counter() - t0)
+            runner.free_request("p")
+        pf = min(times[1:])
+        prefill = {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS,
+                   "ms": round(pf * 1e3, 3),
+                   "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pf / PEAK_FLOPS[args.dtype], 4)}
+
+    line = {
+        "metric": "decode tok/s (Qwen3-8B shape, random weights)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": "Qwen3-8B shape", "layers": args.layers, "layers_full": FULL_LAYERS,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
+                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate": cfg.intermediate_size, "vocab": V, "global_batch": args.batch,
+                   "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": PAGE,
+                   "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
+                   "weights": "random N(0,0.02)"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if prefill:
+        line["prefill"] = prefill
+    if points:
+        points[f"decode_b{args.batch}"] = round(value, 1)
+        line["points"] = points
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -173,13 +173,14 @@ def test_linear(ops, dtype, out_dtype, M, N, K):
 
 
 def test_linear_fp32_is_true_fp32(ops):
-    """A product that bf16 or tf32 inputs would get wrong: 1 + 2^-20 squared sums."""
-    K = 512
-    x = torch.full((4, K), 1.0 + 2.0 ** -20, device=DEV)
-    w = torch.full((8, K), 1.0 + 2.0 ** -20, device=DEV)
+    """Inputs 1 + 2^-12 round to 1 in bf16 and tf32; a true 32-bit product keeps the 2^-11 per term."""
+    K = 64
+    x = torch.full((4, K), 1.0 + 2.0 ** -12, device=DEV)
+    w = torch.full((8, K), 1.0 + 2.0 ** -12, device=DEV)
     y = ops.linear(x, w)
-    want = K * (1.0 + 2.0 ** -20) ** 2
-    assert abs(float(y[0, 0]) - want) < 1e-3 * 2.0 ** -10 * K
+    want = K * (1.0 + 2.0 ** -12) ** 2          # 64.03125...
+    assert abs(float(y[0, 0]) - want) < 1e-4
+    assert abs(float(y[3, 7]) - want) < 1e-4
 
 
 def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
