@@ -9,7 +9,8 @@
 // Tables: page_table[cu_pages[s] + i] is the i-th listed page of request s, whose first row
 // holds position kv_start[s]; new tokens of s are rows cu_q[s]..cu_q[s+1]-1 of q and sit at
 // positions q_start[s], q_start[s]+1, ... (rollout/cache.py:282-328 has the same tables
-// with per-page valid counts instead of kv_start).
+// with per-page valid counts instead of kv_start). tok_ids, if given, lists the T_tokens rows
+// of q to work on (the others belong to another kernel).
 #include "common.h"
 
 #define PLAIN_MAX_ACC 8     // D <= 64 * 8
@@ -19,14 +20,16 @@ __global__ __launch_bounds__(64) void attn_plain_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, const int* __restrict__ page_table,
     const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
-    const int* __restrict__ cu_q, const int* __restrict__ q_start, int n_seqs, int Hq, int Hkv,
-    int D, int P, float scale, int window) {
+    const int* __restrict__ cu_q, const int* __restrict__ q_start,
+    const int* __restrict__ tok_ids, int n_seqs, int Hq, int Hkv, int D, int P, float scale,
+    int window) {
     extern __shared__ float smem[];
     float* q_s = smem;                       // [D]
     float* p_s = smem + D;                   // [64]
     int* row_s = (int*)(smem + D + 64);      // [64]
 
-    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int t = tok_ids ? tok_ids[blockIdx.x] : (int)blockIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x;
     int lo = 0, hi = n_seqs - 1;
     while (lo < hi) {
         const int mid = (lo + hi + 1) >> 1;
@@ -103,8 +106,8 @@ __global__ __launch_bounds__(64) void attn_plain_kernel(
 
 extern "C" int ra_attention_plain(const void* q, void* out, const void* k_pool, const void* v_pool,
                                   const int* page_table, const int* cu_pages, const int* kv_start,
-                                  const int* cu_q, const int* q_start, int n_seqs, int T_tokens,
-                                  int Hq, int Hkv, int D, int P, float scale, int window, int dtype,
+                                  const int* cu_q, const int* q_start, const int* tok_ids,
+                                  int n_seqs, int T_tokens, int Hq, int Hkv, int D, int P, float scale, int window, int dtype,
                                   void* stream) {
     if (T_tokens <= 0 || n_seqs <= 0) return RA_OK;
     if (D > 64 * PLAIN_MAX_ACC || D <= 0 || Hkv <= 0 || Hq % Hkv != 0 || P <= 0) return RA_ERR_ARG;
@@ -114,10 +117,12 @@ extern "C" int ra_attention_plain(const void* q, void* out, const void* k_pool, 
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(attn_plain_kernel<float>, grid, block, shmem, st, (const float*)q,
                            (float*)out, (const float*)k_pool, (const float*)v_pool, page_table,
-                           cu_pages, kv_start, cu_q, q_start, n_seqs, Hq, Hkv, D, P, scale, window);
+                           cu_pages, kv_start, cu_q, q_start, tok_ids, n_seqs, Hq, Hkv, D, P, scale,
+                           window);
     else
         hipLaunchKernelGGL(attn_plain_kernel<bf16>, grid, block, shmem, st, (const bf16*)q,
                            (bf16*)out, (const bf16*)k_pool, (const bf16*)v_pool, page_table,
-                           cu_pages, kv_start, cu_q, q_start, n_seqs, Hq, Hkv, D, P, scale, window);
+                           cu_pages, kv_start, cu_q, q_start, tok_ids, n_seqs, Hq, Hkv, D, P, scale,
+                           window);
     return ra_launch_status();
 }

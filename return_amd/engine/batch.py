@@ -54,6 +54,13 @@ class StepBatch:
     all_decode: bool             # every request brings exactly one token
     max_q_len: int
     max_seq_len: int
+    # requests that bring one token go to the decode kernels, the others to the prefill kernels
+    n_decode: int = 0
+    decode_segs: Optional[torch.Tensor] = None     # int32 [n_decode] request numbers; None: all of them
+    max_decode_seq_len: int = 0
+    n_prefill_tokens: int = 0
+    prefill_toks: Optional[torch.Tensor] = None    # int32 token rows of the others; None: all rows
+    prefill_segs: List[int] = dataclasses.field(default_factory=list)   # host: their request numbers
 
 
 class StepBuilder:
@@ -66,7 +73,8 @@ class StepBuilder:
         self.max_requests = int(max_requests)
         T, N, G = self.max_tokens, self.max_requests, len(cache.groups)
         layout = [("token_ids", T), ("positions", T), ("logit_rows", T), ("cu_q", N + 1),
-                  ("q_start", N), ("seq_lens", N), ("slot_ids", N)]
+                  ("q_start", N), ("seq_lens", N), ("slot_ids", N), ("decode_segs", N),
+                  ("prefill_toks", T)]
         for g in range(G):
             layout += [(f"slot_mapping{g}", T), (f"cu_pages{g}", N + 1), (f"kv_start{g}", N)]
         self._small_end = None
@@ -124,6 +132,14 @@ class StepBuilder:
         self._put("q_start", tables.q_start)
         self._put("seq_lens", tables.seq_lens)
         self._put("slot_ids", tables.slot_ids)
+        dec = [i for i, q in enumerate(tables.q_lens) if q == 1]
+        pre = [i for i, q in enumerate(tables.q_lens) if q != 1]
+        mixed_kinds = bool(dec) and bool(pre)
+        n_pre_tok = T - len(dec)
+        if mixed_kinds:
+            self._put("decode_segs", np.asarray(dec, dtype=np.int32))
+            self._put("prefill_toks", np.concatenate(
+                [np.arange(tables.cu_q[i], tables.cu_q[i + 1], dtype=np.int32) for i in pre]))
         for g, gt in enumerate(tables.groups):
             self._put(f"slot_mapping{g}", gt.slot_mapping)
             self._put(f"cu_pages{g}", gt.cu_pages)
@@ -155,4 +171,9 @@ class StepBuilder:
             q_starts=tables.q_start.tolist(), slot_ids_host=tables.slot_ids.tolist(),
             all_decode=all(q == 1 for q in tables.q_lens),
             max_q_len=max(tables.q_lens) if tables.q_lens else 0,
-            max_seq_len=int(tables.seq_lens.max()) if n else 0)
+            max_seq_len=int(tables.seq_lens.max()) if n else 0,
+            n_decode=len(dec), decode_segs=self._view("decode_segs", len(dec)) if mixed_kinds else None,
+            max_decode_seq_len=max((int(tables.seq_lens[i]) for i in dec), default=0),
+            n_prefill_tokens=n_pre_tok,
+            prefill_toks=self._view("prefill_toks", n_pre_tok) if mixed_kinds else None,
+            prefill_segs=pre)

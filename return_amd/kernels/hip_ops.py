@@ -59,7 +59,8 @@ def _declare(lib):
         "ra_qkv_prepare": [P, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, L, I, P],
         "ra_silu_mul": [P, P, I, I, I, P],
         "ra_gemm_nt": [P, P, P, I, I, I, I, I, P],
-        "ra_attention_plain": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
     }
     for name, args in sigs.items():
@@ -83,6 +84,7 @@ class HipOps:
         # float32 products must be true 32-bit wherever a library routine is used
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
+        self.decode_split_tokens = 64        # keys per split of the decode attention (multiple of 64)
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -271,10 +273,31 @@ class HipOps:
         if D > 512:
             raise KernelError(f"attention: head size {D} is beyond the kernel's 512")
         P = k_pool.shape[1]
+        window = int(window)
+        tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
+        fast_decode = (q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
+                       and n_q // n_kv <= 16)
+        if fast_decode:
+            S = self.decode_split_tokens
+            longest = step.max_decode_seq_len
+            max_splits = (longest - 1) // S + 1
+            if window > 0:                       # a window spans at most this many splits
+                max_splits = min(max_splits, (window + S - 2) // S + 1)
+            nd = step.n_decode
+            part_acc = torch.empty(nd, n_q, max_splits, D, dtype=torch.float32, device=self.device)
+            part_ml = torch.empty(nd, n_q, max_splits, 2, dtype=torch.float32, device=self.device)
+            self._check(self.lib.ra_attention_decode_bf16(
+                _ptr(q), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(k_pool), _ptr(v_pool), *tabs,
+                _ptr(step.decode_segs), nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
+                self._stream()), "attention_decode_bf16")
+            if step.n_prefill_tokens == 0:
+                return
+            toks, n_tok = step.prefill_toks, step.n_prefill_tokens
+        else:
+            toks, n_tok = None, T
         self._check(self.lib.ra_attention_plain(
-            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), _ptr(g.page_table), _ptr(g.cu_pages),
-            _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start), step.n_seqs, T, n_q, n_kv, D, P,
-            float(scale), int(window), _code(q.dtype), self._stream()), "attention_plain")
+            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
+            n_q, n_kv, D, P, float(scale), window, _code(q.dtype), self._stream()), "attention_plain")
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, top_p, u):

@@ -196,7 +196,15 @@ def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
     g = types.SimpleNamespace(page_table=i32([p for ps in pages_of for p in ps]), cu_pages=i32(cu_p),
                               kv_start=i32(kv_starts or [0] * n), slot_mapping=None,
                               n_pages=[len(p) for p in pages_of], max_pages=max(len(p) for p in pages_of))
-    return types.SimpleNamespace(n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
+    dec = [i for i, q in enumerate(q_lens) if q == 1]
+    pre = [i for i, q in enumerate(q_lens) if q != 1]
+    both = bool(dec) and bool(pre)
+    extra = dict(n_decode=len(dec), decode_segs=i32(dec) if both else None,
+                 max_decode_seq_len=max([q_starts[i] + 1 for i in dec], default=0),
+                 n_prefill_tokens=cu_q[-1] - len(dec),
+                 prefill_toks=i32([t for i in pre for t in range(cu_q[i], cu_q[i + 1])]) if both else None,
+                 prefill_segs=pre)
+    return types.SimpleNamespace(**extra, n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
                                  seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
                                  q_lens=list(q_lens), q_starts=list(q_starts),
                                  all_decode=all(q == 1 for q in q_lens), max_q_len=max(q_lens),
@@ -213,6 +221,13 @@ ATTN_CASES = [
     (4, 4, 80, 8, [(30, 10), (1, 77)], 12),
     (3, 1, 64, 16, [(64, 64), (1, 128)], 33),
     (2, 1, 256, 16, [(19, 30)], 0),
+    (32, 8, 128, 16, [(1, 2047), (1, 63), (1, 64), (1, 65)], 0),
+    (16, 1, 64, 32, [(1, 300), (1, 5)], 0),
+    (4, 2, 96, 16, [(1, 130), (3, 7), (1, 0)], 0),
+    (8, 2, 208, 16, [(1, 150), (1, 1)], 0),
+    (6, 2, 32, 8, [(1, 400), (1, 77), (5, 70), (1, 3)], 70),
+    (4, 4, 256, 16, [(1, 199)], 0),
+    (24, 1, 64, 16, [(1, 100)], 0),
 ]
 
 
