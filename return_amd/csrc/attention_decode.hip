@@ -2,21 +2,29 @@
 // split along the keys so that a single request still fills the chip.
 //
 // What it restates of the reference: rollout/attention.py:430-514 (_decode_split_kernel: one
-// program per (request, kv head, split) handles the whole GQA group, block of 16 query rows,
-// writes un-normalised partial sums with their running maximum m and sum l) and
+// program per (request, kv head, split) handles the whole GQA group as a block of 16 query
+// rows and writes un-normalised partial sums with their running maximum m and sum l) and
 // rollout/attention.py:517-540 (_decode_combine: log-sum-exp merge of the splits).
 // Different here: keys are already rotated in the cache; splits are fixed runs of
-// `split_tokens` positions (not a share of the pages that depends on batch size as in
-// rollout/attention.py:543-546), so a request's result does not depend on the batch.
+// `split_tokens` positions counted from position 0 (the reference gives every split a share
+// of the pages, rollout/attention.py:458-461).
 //
-// One wave per (request, kv head, split). Scores S^T = K Q^T come from MFMA 16x16x16 bf16
-// with the key tile as the A operand, read straight from the cache: lane (m, g) holds
-// key m's elements d = g*D/4 + 4j .. +3 for MFMA j, and the query operand is laid out the
-// same way, so each lane reads one contiguous quarter of its key row. The result leaves
-// lane (n, g) with the scores of query head n for keys 4g..4g+3 of each 16-key tile.
-// P.V runs on the vector unit: a lane owns a few columns d and walks the 64 keys.
+// One wave per (request, kv head, split), 64 keys per pass.
+//  scores  S^T = K Q^T by MFMA 16x16x32 bf16, the key tile as A operand read straight from
+//          the cache: lane (n, g) loads the 16 bytes d = 32j + 8g .. +7 of key n, so the four
+//          lane groups of a key read 64 contiguous bytes per load. A trailing 16 of D is one
+//          more step of the same MFMA with the upper half of k zero (an accumulation chain
+//          that mixed 16x16x32 and 16x16x16 lost the last 16x16x32 term on gfx950, so one
+//          shape is used throughout). Lane (n, g) ends up with query head n, keys 4g..4g+3
+//          of each tile.
+//  P.V     on the vector unit: D/8 lanes share a key's value row (16 bytes each), so one load
+//          instruction fetches 64/(D/8) keys; every lane accumulates its 8 columns over the
+//          keys it sees, and the lanes' partial sums are added through LDS at the end.
+// BUILD-VARIANTS: DEC_PART=0 DEC_PART=1 DEC_PART=2 DEC_PART=3 DEC_API=1
+// (each DEC_PART instantiates four head sizes; DEC_API holds the entry point and the merge)
 #include "common.h"
 
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
@@ -41,7 +49,13 @@ __device__ __forceinline__ DecodeRange decode_range(int pos_q, int start, int wi
     return r;
 }
 
-template <int D16>
+#ifdef DEC_PART
+union V16 {
+    uint4 u;
+    uint32_t w[4];
+};
+
+template <int D16, int GMAX>
 __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16* __restrict__ q, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
@@ -50,12 +64,16 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     const int* __restrict__ q_start, const int* __restrict__ seg_ids, int Hq, int Hkv, int P,
     float scale, int window, int split_tokens, int max_splits) {
     constexpr int D = 16 * D16;
-    constexpr int VEC = (D % 128 == 0) ? 2 : 1;                 // columns per lane per V load
-    constexpr int NE = (D + 64 * VEC - 1) / (64 * VEC);        // V loads per key per lane
-    constexpr bool PRELOAD_V = (D <= 128);
+    constexpr int D32 = D / 32;                 // full MFMA x32 steps
+    constexpr bool TAIL16 = (D % 32) != 0;      // one more step of 16
+    constexpr int LPR = D / 8;                  // lanes that share one value row
+    constexpr int KPI = 64 / LPR;               // keys per value load instruction
+    constexpr int NVI = (DEC_CHUNK + KPI - 1) / KPI;   // value load instructions per pass
 
-    __shared__ float p_s[DEC_CHUNK * DEC_MAX_GROUP];           // [key][query head]
+    __shared__ float p_s[DEC_CHUNK * DEC_MAX_GROUP];   // [key][query head]
     __shared__ float alpha_s[DEC_MAX_GROUP];
+    __shared__ int row_s[DEC_CHUNK];
+    extern __shared__ float red_s[];                   // [KPI][G][D] at the end
 
     const int di = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
     const int seg = seg_ids ? seg_ids[di] : di;
@@ -68,55 +86,66 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     if (rg.lo > rg.hi) return;
     const int* pt = page_table + cu_pages[seg];
 
-    // query operand: lane (n, g) holds head kvh*G+n, elements g*D/4 + 4j..+3
-    short4_t bq[D16];
+    // query operand: lane (n, g) holds head kvh*G+n, d = 32j + 8g .. +7 (and D-16+4g.. for the tail)
+    const bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8_t bq[D32 > 0 ? D32 : 1];
+    bf16x8_t bq_tail = z8;
     {
-        const bf16* qp = q + ((size_t)t * Hq + (size_t)kvh * G + (n < G ? n : 0)) * D + g * (D / 4);
+        const bf16* qp = q + ((size_t)t * Hq + (size_t)kvh * G + (n < G ? n : 0)) * D;
 #pragma unroll
-        for (int j = 0; j < D16; ++j) {
-            short4_t v = *reinterpret_cast<const short4_t*>(qp + 4 * j);
-            if (n >= G) v = short4_t{0, 0, 0, 0};
-            bq[j] = v;
+        for (int j = 0; j < D32; ++j) {
+            bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(qp + 32 * j + 8 * g);
+            bq[j] = (n < G) ? v : z8;
+        }
+        if constexpr (TAIL16) {
+            if (n < G && g < 2) bq_tail = *reinterpret_cast<const bf16x8_t*>(qp + (D - 16) + 8 * g);
         }
     }
 
+    // value stage: this lane's columns and its key slot within a load instruction
+    const int vkey = lane / LPR, vcol = (lane % LPR) * 8;
+    const bool v_active = lane < KPI * LPR;
+
     float m_run = -INFINITY, l_run = 0.f;
-    float acc[DEC_MAX_GROUP][NE * VEC];
+    float acc[GMAX][8];
 #pragma unroll
-    for (int h = 0; h < DEC_MAX_GROUP; ++h)
+    for (int h = 0; h < GMAX; ++h)
 #pragma unroll
-        for (int e = 0; e < NE * VEC; ++e) acc[h][e] = 0.f;
+        for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
 
     const int c_begin = (rg.lo / DEC_CHUNK) * DEC_CHUNK;
     for (int c0 = c_begin; c0 <= rg.hi; c0 += DEC_CHUNK) {
         // row of this lane's key (clamped into the split so that every address is valid)
-        int kpos = c0 + lane;
-        kpos = min(max(kpos, rg.lo), rg.hi);
+        int kpos = min(max(c0 + lane, rg.lo), rg.hi);
         const int idx = kpos - start;
         const int row = pt[idx / P] * P + idx % P;
+        row_s[lane] = row;
 
         // ---- K tiles straight into MFMA A operands
-        short4_t ak[4][D16];
+        bf16x8_t ak[4][D32 > 0 ? D32 : 1];
+        bf16x8_t ak_tail[4];
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             const int r = __shfl(row, st * 16 + n, 64);
-            const bf16* kp = k_pool + ((size_t)r * Hkv + kvh) * D + g * (D / 4);
+            const bf16* kp = k_pool + ((size_t)r * Hkv + kvh) * D;
 #pragma unroll
-            for (int j = 0; j < D16; ++j) ak[st][j] = *reinterpret_cast<const short4_t*>(kp + 4 * j);
+            for (int j = 0; j < D32; ++j)
+                ak[st][j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
+            if constexpr (TAIL16) {
+                ak_tail[st] = z8;
+                if (g < 2) ak_tail[st] = *reinterpret_cast<const bf16x8_t*>(kp + (D - 16) + 8 * g);
+            }
         }
-        // ---- V rows for the vector stage
-        uint32_t vreg[PRELOAD_V ? DEC_CHUNK : 1][NE];
-        if constexpr (PRELOAD_V) {
+        __syncthreads();                           // row_s visible
+        // ---- V rows: issue all loads of the pass now
+        V16 vv[NVI];
 #pragma unroll
-            for (int k = 0; k < DEC_CHUNK; ++k) {
-                const int r = __builtin_amdgcn_readlane(row, k);
-                const bf16* vp = v_pool + ((size_t)r * Hkv + kvh) * D;
-#pragma unroll
-                for (int e = 0; e < NE; ++e) {
-                    const int d = e * 64 * VEC + lane * VEC;
-                    if (VEC == 2) vreg[k][e] = *reinterpret_cast<const uint32_t*>(vp + d);
-                    else vreg[k][e] = (d < D) ? (uint32_t)vp[d].x : 0u;
-                }
+        for (int i = 0; i < NVI; ++i) {
+            const int k = i * KPI + vkey;
+            vv[i].u = make_uint4(0u, 0u, 0u, 0u);
+            if (v_active && k < DEC_CHUNK) {
+                const int r = row_s[k];
+                vv[i].u = *reinterpret_cast<const uint4*>(v_pool + ((size_t)r * Hkv + kvh) * D + vcol);
             }
         }
 
@@ -127,8 +156,10 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
         for (int st = 0; st < 4; ++st) {
             float4_t c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < D16; ++j)
-                c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ak[st][j], bq[j], c, 0, 0, 0);
+            for (int j = 0; j < D32; ++j)
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[st][j], bq[j], c, 0, 0, 0);
+            if constexpr (TAIL16)
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak_tail[st], bq_tail, c, 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int kp_abs = c0 + st * 16 + 4 * g + i;
@@ -139,7 +170,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);            // finite: the chunk holds a valid key
+        const float m_new = fmaxf(m_run, mx);            // finite: the pass holds a valid key
         float lsum = 0.f;
 #pragma unroll
         for (int st = 0; st < 4; ++st)
@@ -159,66 +190,50 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
 
         // ---- P.V on the vector unit
 #pragma unroll
-        for (int h = 0; h < DEC_MAX_GROUP; ++h) {
-            if (h >= G) break;
+        for (int h = 0; h < GMAX; ++h) {
             const float a = alpha_s[h];
 #pragma unroll
-            for (int e = 0; e < NE * VEC; ++e) acc[h][e] *= a;
+            for (int e = 0; e < 8; ++e) acc[h][e] *= a;
         }
 #pragma unroll
-        for (int k = 0; k < DEC_CHUNK; ++k) {
-            float vf[NE * VEC];
-            if constexpr (PRELOAD_V) {
+        for (int i = 0; i < NVI; ++i) {
+            const int k = i * KPI + vkey;
+            if (v_active && k < DEC_CHUNK) {
+                float vf[8];
 #pragma unroll
-                for (int e = 0; e < NE; ++e) {
-                    if (VEC == 2) {
-                        vf[2 * e] = __uint_as_float(vreg[k][e] << 16);
-                        vf[2 * e + 1] = __uint_as_float(vreg[k][e] & 0xffff0000u);
-                    } else {
-                        vf[e] = __uint_as_float(vreg[k][e] << 16);
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    vf[2 * e] = __uint_as_float(vv[i].w[e] << 16);
+                    vf[2 * e + 1] = __uint_as_float(vv[i].w[e] & 0xffff0000u);
                 }
-            } else {
-                const int r = __builtin_amdgcn_readlane(row, k);
-                const bf16* vp = v_pool + ((size_t)r * Hkv + kvh) * D;
 #pragma unroll
-                for (int e = 0; e < NE; ++e) {
-                    const int d = e * 64 * VEC + lane * VEC;
-                    if (VEC == 2) {
-                        const uint32_t u = *reinterpret_cast<const uint32_t*>(vp + d);
-                        vf[2 * e] = __uint_as_float(u << 16);
-                        vf[2 * e + 1] = __uint_as_float(u & 0xffff0000u);
-                    } else {
-                        vf[e] = (d < D) ? to_f(vp[d]) : 0.f;
-                    }
+                for (int h = 0; h < GMAX; ++h) {
+                    const float p = p_s[k * DEC_MAX_GROUP + h];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
                 }
-            }
-#pragma unroll
-            for (int h = 0; h < DEC_MAX_GROUP; ++h) {
-                if (h >= G) break;
-                const float p = p_s[k * DEC_MAX_GROUP + h];
-#pragma unroll
-                for (int e = 0; e < NE * VEC; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
             }
         }
         __syncthreads();
     }
 
-    // ---- partial results of this split
+    // ---- add the key slots' partial sums through LDS, then write the split's result
+    if (v_active) {
 #pragma unroll
-    for (int h = 0; h < DEC_MAX_GROUP; ++h) {
-        if (h >= G) break;
-        float* pa = part_acc + (((size_t)di * Hq + (size_t)kvh * G + h) * max_splits + sp) * D;
+        for (int h = 0; h < GMAX; ++h) {
+            if (h < G) {
+                float* r = red_s + ((size_t)vkey * G + h) * D + vcol;
 #pragma unroll
-        for (int e = 0; e < NE; ++e) {
-            const int d = e * 64 * VEC + lane * VEC;
-            if (VEC == 2) {
-                pa[d] = acc[h][2 * e];
-                pa[d + 1] = acc[h][2 * e + 1];
-            } else if (d < D) {
-                pa[d] = acc[h][e];
+                for (int e = 0; e < 8; ++e) r[e] = acc[h][e];
             }
         }
+    }
+    __syncthreads();
+    for (int e = lane; e < G * D; e += 64) {
+        float sum = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KPI; ++ks) sum += red_s[(size_t)ks * G * D + e];
+        const int h = e / D, d = e % D;
+        part_acc[(((size_t)di * Hq + (size_t)kvh * G + h) * max_splits + sp) * D + d] = sum;
     }
     if (g == 0 && n < G) {
         float* pm = part_ml + (((size_t)di * Hq + (size_t)kvh * G + n) * max_splits + sp) * 2;
@@ -227,42 +242,103 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     }
 }
 
-// Merge of the splits, in split order: out = sum_s acc_s * exp(m_s - m) / sum_s l_s * exp(m_s - m).
-__global__ __launch_bounds__(64) void attn_decode_combine_kernel(
+template <int D16, int GMAX>
+static void launch_decode(dim3 grid, size_t shmem, hipStream_t st, const bf16* q, float* pa,
+                          float* pm, const bf16* kp, const bf16* vp, const int* pt, const int* cup,
+                          const int* kvs, const int* cuq, const int* qs, const int* segs, int Hq,
+                          int Hkv, int P, float scale, int window, int split_tokens, int max_splits) {
+    hipLaunchKernelGGL((attn_decode_kernel<D16, GMAX>), grid, dim3(64), shmem, st, q, pa, pm, kp, vp,
+                       pt, cup, kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens,
+                       max_splits);
+}
+
+template <int D16>
+static int pick_group(int G, dim3 grid, size_t shmem, hipStream_t st, const bf16* q, float* pa,
+                      float* pm, const bf16* kp, const bf16* vp, const int* pt, const int* cup,
+                      const int* kvs, const int* cuq, const int* qs, const int* segs, int Hq, int Hkv,
+                      int P, float scale, int window, int split_tokens, int max_splits) {
+#define GO(GM)                                                                                     \
+    launch_decode<D16, GM>(grid, shmem, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs, segs, Hq, Hkv, \
+                           P, scale, window, split_tokens, max_splits)
+    if (G <= 4) GO(4);
+    else if (G <= 16) GO(16);
+    else return RA_ERR_ARG;
+#undef GO
+    return RA_OK;
+}
+
+
+#define DEC_CAT2(a, b) a##b
+#define DEC_CAT(a, b) DEC_CAT2(a, b)
+// head sizes 16*(4*DEC_PART+1) .. 16*(4*DEC_PART+4)
+extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, int G, dim3 grid, size_t shmem, hipStream_t st,
+                                              const bf16* q, float* pa, float* pm, const bf16* kp,
+                                              const bf16* vp, const int* pt, const int* cup,
+                                              const int* kvs, const int* cuq, const int* qs,
+                                              const int* segs, int Hq, int Hkv, int P, float scale,
+                                              int window, int split_tokens, int max_splits) {
+#define DEC_CASE(N)                                                                              \
+    case N:                                                                                      \
+        return pick_group<N>(G, grid, shmem, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs, segs, \
+                             Hq, Hkv, P, scale, window, split_tokens, max_splits);
+    switch (D16) {
+        DEC_CASE(4 * DEC_PART + 1) DEC_CASE(4 * DEC_PART + 2) DEC_CASE(4 * DEC_PART + 3)
+        DEC_CASE(4 * DEC_PART + 4)
+        default: return RA_ERR_ARG;
+    }
+#undef DEC_CASE
+}
+#endif  // DEC_PART
+
+#ifdef DEC_API
+
+#define DEC_PART_ARGS int D16, int G, dim3 grid, size_t shmem, hipStream_t st, const bf16* q, float* pa, \
+    float* pm, const bf16* kp, const bf16* vp, const int* pt, const int* cup, const int* kvs,          \
+    const int* cuq, const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,   \
+    int split_tokens, int max_splits
+extern "C" int ra_dec_part_0(DEC_PART_ARGS);
+extern "C" int ra_dec_part_1(DEC_PART_ARGS);
+extern "C" int ra_dec_part_2(DEC_PART_ARGS);
+extern "C" int ra_dec_part_3(DEC_PART_ARGS);
+
+// Merge of the splits, in split order: out = sum_s acc_s * w_s / sum_s l_s * w_s, w_s = exp(m_s - m).
+__global__ __launch_bounds__(128) void attn_decode_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
     const int* __restrict__ kv_start, const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ seg_ids, int Hq, int D, int window, int split_tokens, int max_splits) {
-    const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    extern __shared__ float w_s[];                     // [ns]
+    __shared__ float stat[2];
+    const int di = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
     const int seg = seg_ids ? seg_ids[di] : di;
     const int t = cu_q[seg];
     const DecodeRange rg = decode_range(q_start[seg], kv_start[seg], window, split_tokens, 0);
     const int ns = min(rg.n_splits, max_splits);
     const float* pm = part_ml + ((size_t)di * Hq + head) * max_splits * 2;
     const float* pa = part_acc + ((size_t)di * Hq + head) * max_splits * D;
-    float m = -INFINITY;
-    for (int s = 0; s < ns; ++s) m = fmaxf(m, pm[2 * s]);
-    float l = 0.f;
-    for (int s = 0; s < ns; ++s) l += pm[2 * s + 1] * __expf(pm[2 * s] - m);
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    for (int d = lane; d < D; d += 64) {
+    if (tid < 64) {                                    // first wave: maximum, weights, sum in split order
+        float m = -INFINITY;
+        for (int s = tid; s < ns; s += 64) m = fmaxf(m, pm[2 * s]);
+        m = wave_max(m);
+        for (int s = tid; s < ns; s += 64) w_s[s] = __expf(pm[2 * s] - m);
+        if (tid == 0) {
+            float l = 0.f;
+            for (int s = 0; s < ns; ++s) l += pm[2 * s + 1] * __expf(pm[2 * s] - m);
+            stat[0] = l > 0.f ? 1.0f / l : 0.f;
+        }
+    }
+    __syncthreads();
+    const float inv = stat[0];
+    for (int d = tid; d < D; d += 128) {
         float o = 0.f;
-        for (int s = 0; s < ns; ++s) o += pa[(size_t)s * D + d] * __expf(pm[2 * s] - m);
+#pragma unroll 8
+        for (int s = 0; s < ns; ++s) o = fmaf(pa[(size_t)s * D + d], w_s[s], o);
         out[((size_t)t * Hq + head) * D + d] = from_f<bf16>(o * inv);
     }
 }
 
-template <int D16>
-static void launch_decode(dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm,
-                          const bf16* kp, const bf16* vp, const int* pt, const int* cup,
-                          const int* kvs, const int* cuq, const int* qs, const int* segs, int Hq,
-                          int Hkv, int P, float scale, int window, int split_tokens, int max_splits) {
-    hipLaunchKernelGGL(attn_decode_kernel<D16>, grid, dim3(64), 0, st, q, pa, pm, kp, vp, pt, cup,
-                       kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits);
-}
-
 // part_acc: fp32 [n_dec, Hq, max_splits, D]; part_ml: fp32 [n_dec, Hq, max_splits, 2].
-// max_splits must cover ceil((longest sequence)/split_tokens) + 1 splits... the host passes
-// the number of splits of the longest request; requests with fewer leave the rest untouched.
+// max_splits is the number of splits of the request with the most; requests with fewer leave
+// the rest untouched and the merge does not read it.
 extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc, void* part_ml,
                                         const void* k_pool, const void* v_pool,
                                         const int* page_table, const int* cu_pages,
@@ -277,26 +353,29 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(n_dec, Hkv, max_splits);
+    const int G = Hq / Hkv;
+    const int kpi = 64 / (D / 8);
+    const size_t shmem = (size_t)kpi * G * D * sizeof(float);
+    if (shmem > 48 * 1024) return RA_ERR_ARG;
     const bf16* qq = (const bf16*)q;
     const bf16* kp = (const bf16*)k_pool;
     const bf16* vp = (const bf16*)v_pool;
     float* pa = (float*)part_acc;
     float* pm = (float*)part_ml;
-#define DEC_CASE(N)                                                                              \
-    case N:                                                                                      \
-        launch_decode<N>(grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q,     \
-                         q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); \
-        break;
-    switch (D / 16) {
-        DEC_CASE(1) DEC_CASE(2) DEC_CASE(3) DEC_CASE(4) DEC_CASE(5) DEC_CASE(6) DEC_CASE(7) DEC_CASE(8)
-        DEC_CASE(9) DEC_CASE(10) DEC_CASE(11) DEC_CASE(12) DEC_CASE(13) DEC_CASE(14) DEC_CASE(15)
-        DEC_CASE(16)
+    int rc;
+    const int d16 = D / 16;
+    switch ((d16 - 1) / 4) {
+        case 0: rc = ra_dec_part_0(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 1: rc = ra_dec_part_1(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 2: rc = ra_dec_part_2(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 3: rc = ra_dec_part_3(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
         default: return RA_ERR_ARG;
     }
-#undef DEC_CASE
+    if (rc != RA_OK) return rc;
     if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
-    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(64), 0, st, pa, pm,
-                       (bf16*)out, kv_start, cu_q, q_start, seg_ids, Hq, D, window, split_tokens,
-                       max_splits);
+    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128),
+                       (size_t)max_splits * sizeof(float), st, pa, pm, (bf16*)out, kv_start, cu_q,
+                       q_start, seg_ids, Hq, D, window, split_tokens, max_splits);
     return ra_launch_status();
 }
+#endif  // DEC_API

@@ -38,6 +38,25 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def compile_units():
+    """(source, defines, object name): a source with a line '// BUILD-VARIANTS: A=1 B=2 ...' is
+    compiled once per listed define (large template families are split to compile in parallel)."""
+    units = []
+    for src in sources():
+        base = os.path.basename(src)[:-4]
+        variants = []
+        with open(src) as f:
+            for line in f:
+                if line.startswith("// BUILD-VARIANTS:"):
+                    variants = line.split(":", 1)[1].split()
+                    break
+        if not variants:
+            units.append((src, [], base + ".o"))
+        for v in variants:
+            units.append((src, ["-D" + v], f"{base}.{v.replace('=', '_')}.o"))
+    return units
+
+
 def _headers():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h"))
 
@@ -107,9 +126,9 @@ def build(force: bool = True) -> str:
     out_dir = _writable_dir()
     obj_dir = os.path.join(out_dir, "_build")
     os.makedirs(obj_dir, exist_ok=True)
-    srcs = sources()
+    units = compile_units()
     t0 = time.time()
-    _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
+    _say(f"compiling {len(units)} HIP units for {ARCH} into {out_dir}")
     done = threading.Event()
 
     def heartbeat():
@@ -118,14 +137,15 @@ def build(force: bool = True) -> str:
 
     threading.Thread(target=heartbeat, daemon=True).start()
     try:
-        def one(src):
-            obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
-            _run([hipcc, *FLAGS, "-c", src, "-o", obj], f"compiling {os.path.basename(src)}")
-            _say(f"compiled {os.path.basename(src)} ({time.time() - t0:.0f} s)")
+        def one(unit):
+            src, defines, name = unit
+            obj = os.path.join(obj_dir, name)
+            _run([hipcc, *FLAGS, *defines, "-c", src, "-o", obj], f"compiling {name}")
+            _say(f"compiled {name[:-2]} ({time.time() - t0:.0f} s)")
             return obj
-        workers = min(len(srcs), max(1, min(8, os.cpu_count() or 1)))
+        workers = min(len(units), max(1, min(8, os.cpu_count() or 1)))
         with concurrent.futures.ThreadPoolExecutor(workers) as pool:
-            objs = list(pool.map(one, srcs))
+            objs = list(pool.map(one, units))
         tmp = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
         _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], "linking")
         lib = os.path.join(out_dir, LIB_NAME)

@@ -59,6 +59,7 @@ def _declare(lib):
         "ra_qkv_prepare": [P, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, L, I, P],
         "ra_silu_mul": [P, P, I, I, I, P],
         "ra_gemm_nt": [P, P, P, I, I, I, I, I, P],
+        "ra_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
@@ -84,7 +85,17 @@ class HipOps:
         # float32 products must be true 32-bit wherever a library routine is used
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
-        self.decode_split_tokens = 64        # keys per split of the decode attention (multiple of 64)
+        self.decode_split_tokens = 0         # keys per split of the decode attention; 0: by batch size
+        self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
+
+    def use_skinny(self, M, N, K, out_dtype):
+        """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
+        (measured on MI355X: it wins for one to four rows, and up to 16 rows on small weights)."""
+        if K % 8 or M > 64:
+            return False
+        if out_dtype == torch.float32:
+            return True                      # the library has no bf16-in, fp32-out product
+        return M <= 4 or (M <= 16 and N * K <= (32 << 20))
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -251,6 +262,11 @@ class HipOps:
         if w.shape[1] != K:
             raise KernelError(f"linear: x {tuple(x.shape)} times weight {tuple(w.shape)}^T")
         out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.bfloat16 and M > 0 and self.use_skinny(M, N, K, out_dtype):
+            y = torch.empty(M, N, dtype=out_dtype, device=self.device)
+            self._check(self.lib.ra_gemm_skinny_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
+                                                     self.skinny_max_grid, self._stream()), "gemm_skinny")
+            return y
         if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and M > 0:
             return torch.matmul(x, w.t())          # library product, as the reference's F.linear
         y = torch.empty(M, N, dtype=out_dtype, device=self.device)
@@ -278,8 +294,12 @@ class HipOps:
         fast_decode = (q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
                        and n_q // n_kv <= 16)
         if fast_decode:
-            S = self.decode_split_tokens
             longest = step.max_decode_seq_len
+            S = self.decode_split_tokens
+            if S <= 0:
+                # enough splits to fill the chip, few enough to keep the merge cheap
+                chunks = step.n_decode * n_kv * ((longest + 63) // 64)
+                S = 64 * max(1, min(8, chunks // 4096))
             max_splits = (longest - 1) // S + 1
             if window > 0:                       # a window spans at most this many splits
                 max_splits = min(max_splits, (window + S - 2) // S + 1)

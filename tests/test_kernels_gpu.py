@@ -253,6 +253,27 @@ def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
     torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("D", list(range(16, 257, 16)))
+def test_decode_attention_every_head_size(ops, ref, D):
+    """The bfloat16 decode kernel at every head size it takes, grouped and ungrouped."""
+    for Hq, Hkv in ((4, 1), (3, 3), (16, 2)):
+        P = 16
+        segs = [(1, 150), (1, 1), (1, 64)]
+        need = [-(-(a + b) // P) for b, a in segs]
+        pages_of, nxt = [], 0
+        for k in need:
+            pages_of.append(list(range(nxt, nxt + k)))
+            nxt += k
+        step = _step([1, 1, 1], [s[1] for s in segs], P, pages_of)
+        kp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D)
+        vp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D + 1)
+        q = rnd(3, Hq, D, dtype=torch.bfloat16, seed=D + 2)
+        a, b = torch.zeros_like(q), torch.zeros_like(q)
+        ops.attention(q, a, kp, vp, step, 0, D ** -0.5, 0)
+        ref.attention(q, b, kp, vp, step, 0, D ** -0.5, 0)
+        torch.testing.assert_close(a.float(), b.float(), **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_far_key_stands_out(ops, dtype):
     """One key far back among hundreds is made to dominate: the output must be its value."""
