@@ -1,0 +1,192 @@
+"""The cache manager on the CPU: no page lost, held twice or freed twice, under random orders
+of requests; tables against a brute-force builder; windows give pages back; reuse is immediate."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from return_amd.cache import CacheManager, FreeList, KVCapacityError, PagedKVSpec, StateSpec
+
+
+def manager(page=4, max_token=64, max_requests=4, window=None, extra=None):
+    layers = {0: PagedKVSpec(2, 8), 1: PagedKVSpec(2, 8)}
+    if window:
+        layers[2] = PagedKVSpec(2, 8, window)
+    if extra:
+        layers.update(extra)
+    return CacheManager(layers, page, max_token, max_requests, torch.float32, "cpu")
+
+
+def test_free_list_refuses_double_free_and_strangers():
+    f = FreeList(3)
+    a, b = f.take(), f.take()
+    f.give_back([a])
+    with pytest.raises(ValueError, match="twice"):
+        f.give_back([a])
+    with pytest.raises(ValueError, match="exist"):
+        f.give_back([7])
+    assert f.take() == a                      # last freed, first reused (rollout/cache.py:153)
+    f.take()
+    with pytest.raises(KVCapacityError):
+        f.take()
+    with pytest.raises(KVCapacityError):
+        FreeList(2).take_many(3)
+
+
+def brute_tables(cm, entries, before):
+    """Tables from the manager's page lists alone (after check_tables.py:11-31 of the reference)."""
+    P = cm.page_size
+    out = []
+    for g in range(len(cm.groups)):
+        slot, table, cu, starts = [], [], [0], []
+        for rid, n in entries:
+            r = cm.live[rid]
+            for pos in range(before[rid], before[rid] + n):
+                rel = pos - r.first_pos[g]
+                slot.append(r.pages[g][rel // P] * P + rel % P)
+            table += r.pages[g]
+            cu.append(len(table))
+            starts.append(r.first_pos[g])
+        out.append((slot, table, cu, starts))
+    return out
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("window", [None, 6])
+def test_random_requests_keep_every_page_accounted(seed, window):
+    rng = random.Random(seed)
+    cm = manager(page=4, max_token=96, max_requests=4, window=window)
+    live, next_id, refused = {}, 0, 0
+    for _ in range(300):
+        op = rng.random()
+        if op < 0.25 and len(live) < 4:
+            cm.add_request(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif op < 0.35 and live:
+            rid = rng.choice(list(live))
+            cm.free_request(rid)
+            del live[rid]
+        elif live:
+            ids = rng.sample(list(live), rng.randint(1, len(live)))
+            entries = [(rid, rng.choice([1, 1, 1, 2, 3, 7, 13])) for rid in ids]
+            before = dict(live)
+            free_before = cm.free_pages()
+            try:
+                t = cm.begin_step(entries)
+            except KVCapacityError:
+                refused += 1
+                assert cm.free_pages() == free_before          # nothing changed
+                assert all(cm.seq_len(r) == before[r] for r in live)
+                cm.check_invariants()
+                continue
+            for rid, n in entries:
+                live[rid] += n
+            want = brute_tables(cm, entries, before)
+            for g, (slot, table, cu, starts) in enumerate(want):
+                assert t.groups[g].slot_mapping.tolist() == slot
+                assert t.groups[g].page_table.tolist() == table
+                assert t.groups[g].cu_pages.tolist() == cu
+                assert t.groups[g].kv_start.tolist() == starts
+            assert t.q_start.tolist() == [before[r] for r, _ in entries]      # tokens held before
+            assert t.seq_lens.tolist() == [live[r] for r, _ in entries]
+            assert t.positions.tolist() == [p for r, n in entries for p in range(before[r], before[r] + n)]
+            assert len(set(t.groups[0].slot_mapping.tolist())) == len(t.groups[0].slot_mapping)
+            cm.end_step()
+        cm.check_invariants()
+    assert refused > 0                                      # the pool was small enough to run out
+    for rid in list(live):
+        cm.free_request(rid)
+    cm.check_invariants()
+    assert all(g.pages.in_use() == 0 for g in cm.groups) and cm.slots.in_use() == 0
+
+
+def test_positions_follow_the_reference_layout():
+    """65 tokens, then 3 more: the second portion starts at position 65 on the second page
+    (qpos = seqlen - q_len, rollout/cache.py:293; vector [0, 65, ...] of opd/test_parallel.py:113)."""
+    cm = CacheManager({0: PagedKVSpec(1, 8)}, 64, 64 * 4, 2, torch.float32, "cpu")
+    cm.add_request("u")
+    t = cm.begin_step([("u", 65)])
+    assert t.q_start.tolist() == [0] and len(cm.live["u"].pages[0]) == 2
+    cm.end_step()
+    t = cm.begin_step([("u", 3)])
+    assert t.q_start.tolist() == [65] and t.positions.tolist() == [65, 66, 67]
+    p = cm.live["u"].pages[0]
+    assert t.groups[0].slot_mapping.tolist() == [p[1] * 64 + 1, p[1] * 64 + 2, p[1] * 64 + 3]
+
+
+def test_pages_are_reused_at_once():
+    cm = manager(page=4, max_token=16, max_requests=2)
+    cm.add_request("a")
+    cm.begin_step([("a", 16)]); cm.end_step()
+    held = list(cm.live["a"].pages[0])
+    cm.add_request("b")
+    with pytest.raises(KVCapacityError):
+        cm.begin_step([("b", 1)])
+    cm.free_request("a")
+    cm.begin_step([("b", 16)]); cm.end_step()
+    assert sorted(cm.live["b"].pages[0]) == sorted(held)
+    with pytest.raises(ValueError, match="not live"):
+        cm.free_request("a")
+
+
+def test_window_gives_pages_back_while_running():
+    cm = manager(page=4, max_token=64, max_requests=2, window=6)
+    g = [i for i, grp in enumerate(cm.groups) if grp.spec.window == 6][0]
+    full = 1 - g
+    cm.add_request("w")
+    held = []
+    for _ in range(40):
+        cm.begin_step([("w", 1)]); cm.end_step()
+        r = cm.live["w"]
+        held.append(len(r.pages[g]))
+        # every key a later query may read is still there
+        assert r.first_pos[g] <= max(0, r.seq_len - 6 + 1)
+        assert r.first_pos[g] + len(r.pages[g]) * 4 >= r.seq_len
+        cm.check_invariants()
+    assert max(held) <= 3 and len(cm.live["w"].pages[full]) == 10
+    cm.add_request("x")
+    cm.begin_step([("x", 24)]); cm.end_step()          # a long portion, then the window trims it
+    assert len(cm.live["x"].pages[g]) <= 3 and cm.live["x"].first_pos[g] == 16
+    assert cm.max_pages(40, 24)[g] >= 24 // 4
+
+
+def test_state_slots():
+    spec = StateSpec((("conv", (3, 2), "bfloat16"), ("rec", (2, 4, 4), "float32")))
+    cm = manager(extra={5: spec}, max_requests=2)
+    s0 = cm.add_request("a")
+    view = cm.view(5)
+    assert view.tensors["rec"].shape == (2, 2, 4, 4) and view.tensors["conv"].dtype == torch.bfloat16
+    view.tensors["rec"][s0] += 3.0
+    cm.add_request("b")
+    with pytest.raises(KVCapacityError):
+        cm.add_request("c")
+    cm.free_request("a")
+    s2 = cm.add_request("c")
+    assert s2 == s0 and float(cm.view(5).tensors["rec"][s2].abs().sum()) == 0.0    # zero at the start
+    t = cm.begin_step([("c", 2), ("b", 1)])
+    assert t.slot_ids.tolist() == [cm.slot_of("c"), cm.slot_of("b")]
+
+
+def test_step_rules():
+    cm = manager()
+    cm.add_request("a")
+    with pytest.raises(ValueError, match="twice"):
+        cm.begin_step([("a", 1), ("a", 1)])
+    with pytest.raises(ValueError, match="not live"):
+        cm.begin_step([("zz", 1)])
+    with pytest.raises(ValueError, match="at least one"):
+        cm.begin_step([("a", 0)])
+    with pytest.raises(ValueError, match="already live"):
+        cm.add_request("a")
+
+
+def test_groups_have_pools_of_their_own():
+    cm = CacheManager({0: PagedKVSpec(2, 8), 1: PagedKVSpec(2, 8, 4), 2: PagedKVSpec(1, 16), 3: PagedKVSpec(2, 8)},
+                      4, 32, 2, torch.float32, "cpu")
+    assert len(cm.groups) == 3
+    assert sorted(map(tuple, (g.layers for g in cm.groups))) == [(0, 3), (1,), (2,)]
+    v0, v3 = cm.view(0), cm.view(3)
+    assert v0.group == v3.group and v0.k_pool.data_ptr() != v3.k_pool.data_ptr()
+    assert v0.k_pool.shape == (8, 4, 2, 8) and cm.view(2).k_pool.shape == (8, 4, 1, 16)

@@ -1,0 +1,93 @@
+"""The engine's host side (cache, step function, scheduler, entry point) on the CPU, with the
+torch stand-in kernels of tests/torch_ops.py in place of the HIP library: every way of cutting
+the work gives the plain implementation's logits, and generation does not depend on the knobs."""
+import pytest
+import torch
+
+from return_amd import SamplingParams
+from return_amd.config import EngineConfig
+from return_amd.engine import Engine, ModelRunner
+from tests import trace_tools as tt
+from tests.conftest import TINY_A, TINY_B
+from tests.plain import qwen3_plain as plain
+from tests.torch_ops import TorchOps
+
+
+def runner_for(folder, max_token, page=16, max_reside=4, **kw):
+    ec = EngineConfig(dtype="float32", page_size=page, max_token=max_token, max_reside=max_reside,
+                      max_step_tokens=max(max_token, max_reside), prefill_chunk=max_token, device="cpu", **kw)
+    return ModelRunner(folder, engine_config=ec, ops=TorchOps())
+
+
+@pytest.mark.parametrize("which", ["a", "b"])
+@pytest.mark.parametrize("cut", ["whole", "tail_decoded", "portions", "mixed"])
+def test_every_cut_matches_plain(which, cut, folder_a, folder_b):
+    folder, raw = (folder_a, TINY_A) if which == "a" else (folder_b, TINY_B)
+    reqs = {rid: tt.random_tokens(raw["vocab_size"], n, seed=ord(rid))
+            for rid, n in {"a": 5, "b": 17, "c": 33, "d": 70, "e": 64, "g": 1}.items()}
+    cfg, w = plain.read_folder(folder)
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    steps = {"whole": tt.whole, "tail_decoded": tt.tail_decoded, "portions": tt.portions, "mixed": tt.mixed}[cut](reqs)
+    runner = runner_for(folder, tt.peak_tokens(steps))
+    got = tt.run_in_process(runner, steps)
+    for rid, toks in reqs.items():
+        for p in range(len(toks)):
+            torch.testing.assert_close(got[(rid, p)], want[rid][p], atol=2e-5, rtol=1e-4)
+    assert all(g.pages.in_use() == 0 for g in runner.cache.groups)
+
+
+def test_generation_does_not_depend_on_the_knobs(folder_b):
+    cfg, w = plain.read_folder(folder_b)
+    prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (1, 8, 31, 64, 100)]
+    want = [plain.greedy_generate(cfg, w, p, 6) for p in prompts]
+    for max_reside, chunk, max_token, page in ((4, 24, 1024, 32), (1, 1000, 256, 16), (5, 7, 416, 8)):
+        ec = EngineConfig(dtype="float32", page_size=page, max_token=max_token, max_reside=max_reside,
+                          max_step_tokens=64, prefill_chunk=chunk, device="cpu")
+        eng = Engine(runner=ModelRunner(folder_b, engine_config=ec, ops=TorchOps()))
+        got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=6))
+        assert [r.output_ids for r in got] == want
+        assert all(r.finish_reason == "length" and r.num_tokens == 6 for r in got)
+        for r, p in zip(got, prompts):                 # logprob is of the raw logits (rollout/model.py:64-67)
+            lp = plain.chosen_logprob(plain.logits(cfg, w, p)[-1], r.output_ids[0])
+            assert abs(r.output_logprobs[0] - lp) < 1e-4
+        eng.runner.cache.check_invariants()
+        assert not eng.runner.cache.live
+
+
+def test_temperature_sampling_is_reproducible_and_batch_independent(folder_a):
+    prompts = [tt.random_tokens(TINY_A["vocab_size"], n, seed=n) for n in (5, 17, 33)]
+    sp = [SamplingParams(temperature=0.7, max_new_tokens=10, seed=100 + i) for i in range(3)]
+    def run(max_reside):
+        ec = EngineConfig(dtype="float32", page_size=16, max_token=512, max_reside=max_reside,
+                          max_step_tokens=64, prefill_chunk=24, device="cpu", seed=7)
+        return [r.output_ids for r in Engine(runner=ModelRunner(folder_a, engine_config=ec, ops=TorchOps()))
+                .generate(prompts, sp)]
+    together, alone = run(3), run(1)
+    assert together == alone == run(3)
+    assert len({tuple(x) for x in together}) == 3
+
+
+def test_stop_sequence_through_the_entry_point(folder_a):
+    cfg, w = plain.read_folder(folder_a)
+    prompt = tt.random_tokens(TINY_A["vocab_size"], 9, seed=4)
+    free = plain.greedy_generate(cfg, w, prompt, 8)
+    eng = Engine(runner=runner_for(folder_a, 256))
+    r = eng.generate([prompt], SamplingParams(temperature=0.0, max_new_tokens=8, stop_ids=[free[2:4]]))[0]
+    want = plain.greedy_generate(cfg, w, prompt, 8, stop_ids=[free[2:4]])
+    assert r.output_ids == want and len(want) < 8 and r.finish_reason == "stop"
+
+
+def test_step_checks(folder_a):
+    from return_amd.engine import StepEntry
+    runner = runner_for(folder_a, 64)
+    runner.add_request("a")
+    with pytest.raises(ValueError, match="vocabulary"):
+        runner.step([StepEntry("a", [TINY_A["vocab_size"]], [0])])
+    with pytest.raises(ValueError, match="not among"):
+        runner.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(ValueError, match="no tokens"):
+        runner.step([StepEntry("a", [], [])])
+    assert runner.step([StepEntry("a", [1, 2, 3], [])]) is None          # nothing wanted, cache still filled
+    assert runner.cache.seq_len("a") == 3
+    with pytest.raises(ValueError, match="max_position"):
+        runner.step([StepEntry("a", [1] * 300, [])])
