@@ -50,6 +50,7 @@ class StepBatch:
     request_ids: List
     q_lens: List[int]
     q_starts: List[int]
+    cu_q_host: List[int]
     slot_ids_host: List[int]
     all_decode: bool             # every request brings exactly one token
     max_q_len: int
@@ -168,7 +169,8 @@ class StepBuilder:
             seq_lens=self._view("seq_lens", n), slot_ids=self._view("slot_ids", n),
             logit_rows=self._view("logit_rows", m), n_logit_rows=m, groups=groups,
             request_ids=list(tables.request_ids), q_lens=list(tables.q_lens),
-            q_starts=tables.q_start.tolist(), slot_ids_host=tables.slot_ids.tolist(),
+            q_starts=tables.q_start.tolist(), cu_q_host=tables.cu_q.tolist(),
+            slot_ids_host=tables.slot_ids.tolist(),
             all_decode=all(q == 1 for q in tables.q_lens),
             max_q_len=max(tables.q_lens) if tables.q_lens else 0,
             max_seq_len=int(tables.seq_lens.max()) if n else 0,

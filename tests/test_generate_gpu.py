@@ -1,0 +1,112 @@
+"""Generation through the entry points on the GPU: greedy equals the plain implementation,
+temperature sampling is reproducible, the command line answers in the reference's fields."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from return_amd import SamplingParams
+from tests import trace_tools as tt
+from tests.conftest import TINY_A, TINY_B
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_greedy_matches_plain_fp32(folder_a, folder_b):
+    from return_amd.engine import Engine
+    for folder, raw, lens, page in ((folder_a, TINY_A, (5, 17, 33), 16), (folder_b, TINY_B, (1, 8, 31, 64, 100), 32)):
+        cfg, w = plain.read_folder(folder)
+        prompts = [tt.random_tokens(raw["vocab_size"], n, seed=n) for n in lens]
+        want = [plain.greedy_generate(cfg, w, p, 16) for p in prompts]
+        eng = Engine(folder, dtype="float32", page_size=page, max_token=2048, max_reside=4,
+                     max_step_tokens=64, prefill_chunk=24)
+        got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=16))
+        assert [r.output_ids for r in got] == want
+        for r, p in zip(got, prompts):
+            seq = p + r.output_ids
+            lg = plain.logits(cfg, w, seq[:-1])
+            for i, (tok, lp) in enumerate(zip(r.output_ids, r.output_logprobs)):
+                assert abs(lp - plain.chosen_logprob(lg[len(p) - 1 + i], tok)) < 2e-4
+        assert not eng.runner.cache.live
+
+
+def test_bf16_generation_follows_plain_within_rounding(folder_b):
+    """bfloat16 may flip near-ties; every sampled token must still be one the plain model finds
+    nearly as likely as its own choice, and the logprobs must agree within bf16 rounding."""
+    from return_amd.engine import Engine
+    cfg, w = plain.read_folder(folder_b)
+    prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (8, 31, 64)]
+    eng = Engine(folder_b, dtype="bfloat16", page_size=16, max_token=2048, max_reside=4)
+    got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=12))
+    for r, p in zip(got, prompts):
+        seq = p + r.output_ids
+        lg = plain.logits(cfg, w, seq[:-1])
+        for i, (tok, lp) in enumerate(zip(r.output_ids, r.output_logprobs)):
+            row = lg[len(p) - 1 + i].double().log_softmax(-1)
+            assert float(row.max() - row[tok]) < 0.05, "sampled a token the plain model finds unlikely"
+            assert abs(lp - float(row[tok])) < 0.05
+
+
+def test_temperature_sampling_reproducible(folder_b):
+    from return_amd.engine import Engine
+    prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (1, 8, 31, 64, 100)]
+    sp = [SamplingParams(temperature=0.7, max_new_tokens=20, seed=50 + i) for i in range(5)]
+    def run(max_reside, chunk):
+        eng = Engine(folder_b, dtype="float32", page_size=32, max_token=4096, max_reside=max_reside,
+                     max_step_tokens=64, prefill_chunk=chunk, seed=11)
+        return [r.output_ids for r in eng.generate(prompts, sp)]
+    a, b = run(5, 24), run(2, 1000)
+    assert a == b and all(len(x) == 20 for x in a)
+
+
+def test_top_k_top_p_through_the_engine(folder_a):
+    from return_amd.engine import Engine
+    cfg, w = plain.read_folder(folder_a)
+    prompt = tt.random_tokens(TINY_A["vocab_size"], 12, seed=2)
+    eng = Engine(folder_a, dtype="float32", page_size=16, max_token=1024, max_reside=4)
+    greedy = eng.generate([prompt], SamplingParams(temperature=0.0, max_new_tokens=6))[0].output_ids
+    k1 = eng.generate([prompt], SamplingParams(temperature=1.5, top_k=1, max_new_tokens=6))[0].output_ids
+    p0 = eng.generate([prompt], SamplingParams(temperature=1.5, top_p=0.0, max_new_tokens=6))[0].output_ids
+    assert greedy == k1 == p0 == plain.greedy_generate(cfg, w, prompt, 6)
+    # with top_k=3 every token is among the plain model's three most likely
+    r = eng.generate([prompt], SamplingParams(temperature=2.0, top_k=3, max_new_tokens=10, seed=5))[0]
+    seq = prompt + r.output_ids
+    lg = plain.logits(cfg, w, seq[:-1])
+    for i, tok in enumerate(r.output_ids):
+        assert tok in lg[len(prompt) - 1 + i].topk(3).indices.tolist()
+
+
+def test_command_line(folder_a, tmp_path):
+    cfg, w = plain.read_folder(folder_a)
+    reqs = [{"session_id": "s0", "prompt_ids": tt.random_tokens(256, 9, seed=1), "max_new_tokens": 5, "temperature": 0.0},
+            {"session_id": "s1", "prompt_ids": tt.random_tokens(256, 20, seed=2), "max_new_tokens": 3, "temperature": 0.0,
+             "stop_ids": [[999]], "top_k": 0, "top_p": 1.0}]
+    f = tmp_path / "reqs.jsonl"
+    f.write_text("\n".join(json.dumps(r) for r in reqs))
+    out = subprocess.run([sys.executable, "-m", "return_amd.cli", "generate", "--model", folder_a, "--dtype", "float32",
+                          "--max-reside", "4", "--max-token", "1024", "--requests", str(f)],
+                         cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    lines = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    assert [l["session_id"] for l in lines] == ["s0", "s1"]
+    for l, r in zip(lines, reqs):
+        assert set(l) == {"session_id", "output_ids", "output_logprobs", "num_tokens", "finish_reason"}
+        assert l["output_ids"] == plain.greedy_generate(cfg, w, r["prompt_ids"], r["max_new_tokens"])
+        assert l["finish_reason"] == "length" and l["num_tokens"] == r["max_new_tokens"]
+    bad = subprocess.run([sys.executable, "-m", "return_amd.cli", "generate", "--model", folder_a, "--requests", "-"],
+                         cwd=ROOT, input=json.dumps({"prompt_ids": [1], "swap": [3], "swap_at": 0}), capture_output=True,
+                         text=True, timeout=300)
+    assert bad.returncode != 0 and "paragraph" in bad.stderr
+
+
+def test_the_library_is_the_one_that_runs():
+    """The HIP library is loaded in this process; there is nothing else behind the kernels."""
+    from return_amd.kernels.hip_ops import HipOps
+    HipOps("cuda:0")
+    with open("/proc/self/maps") as f:
+        assert "libreturn_amd.so" in f.read()

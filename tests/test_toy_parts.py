@@ -1,0 +1,259 @@
+"""Generality of the parts: a toy architecture, defined here and registered through the public
+registries only, with
+  - a mixer that keeps state of its own (an exponential moving average per request),
+  - a feed-forward with routing (top-1 of two experts, router logits in 32-bit),
+  - a position encoding that is no rotation (keys scaled by their position),
+  - a windowed attention layer (pages of its own, given back as the window passes),
+  - a run order that calls one block twice and lets one layer read another layer's cache.
+It is built and stepped without a change to the framework's files and compared, in 32-bit,
+with a dense whole-sequence evaluation written below. This toy is no model of anyone's."""
+import dataclasses
+
+import pytest
+import torch
+
+from return_amd.cache.spec import StateSpec
+from return_amd.config import EngineConfig, ModelConfig, register_architecture
+from return_amd.engine import ModelRunner
+from return_amd.parts import BlockSpec, LayerCall, ModelSpec, PartSpec, register_part
+from return_amd.weights import random_weights
+from tests import trace_tools as tt
+from tests.plain import qwen3_plain as plain
+
+
+# ------------------------------------------------------------------ toy parts (torch on whatever device)
+class EmaMixer:
+    """s_t = decay * s_{t-1} + W x_t ; y_t = s_t. The state lives in the cache manager's slots."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        return {"w": (params["hidden_size"], params["hidden_size"])}
+
+    @staticmethod
+    def random_init(params, role):
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt, self.decay, self.h = rt, float(params["decay"]), int(params["hidden_size"])
+        self.w = rt.matrix(tensors["w"])
+
+    def cache_spec(self):
+        return StateSpec((("s", (self.h,), "float32"),))
+
+    def forward(self, x, step, cache, write_cache=True):
+        u = self.rt.ops.linear(x, self.w).float()
+        y = torch.empty_like(u)
+        for i in range(step.n_seqs):
+            a, b = step.cu_q_host[i], step.cu_q_host[i + 1]
+            s = cache.tensors["s"][step.slot_ids_host[i]].clone()
+            for t in range(a, b):
+                s = self.decay * s + u[t]
+                y[t] = s
+            cache.tensors["s"][step.slot_ids_host[i]] = s
+        return y.to(x.dtype)
+
+
+class RoutedFeedForward:
+    """y = expert_e(x) for e = argmax(router(x)); expert = relu(x W1_e^T) W2_e^T."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        H, I, E = params["hidden_size"], params["intermediate_size"], params["experts"]
+        shapes = {"router": (E, H)}
+        for e in range(E):
+            shapes[f"w1_{e}"] = (I, H)
+            shapes[f"w2_{e}"] = (H, I)
+        return shapes
+
+    @staticmethod
+    def random_init(params, role):
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt, self.E = rt, int(params["experts"])
+        self.router = tensors["router"].to(rt.device).float()
+        self.w1 = [rt.matrix(tensors[f"w1_{e}"]) for e in range(self.E)]
+        self.w2 = [rt.matrix(tensors[f"w2_{e}"]) for e in range(self.E)]
+
+    def forward(self, x, step=None):
+        choice = (x.float() @ self.router.t()).argmax(-1)
+        y = torch.zeros_like(x)
+        for e in range(self.E):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                hid = self.rt.ops.linear(x[rows].contiguous(), self.w1[e]).relu()
+                y[rows] = self.rt.ops.linear(hid.contiguous(), self.w2[e])
+        return y
+
+
+class KeyFade:
+    """Not a rotation: keys are scaled by 1 / (1 + position / horizon). No tables(), so the
+    attention part takes its general path (norm, apply(), cache write)."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        return {}
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.horizon = float(params["horizon"])
+
+    def apply(self, q, k, positions):
+        if k is not None:
+            k.mul_((1.0 / (1.0 + positions.float() / self.horizon)).to(k.dtype)[:, None, None])
+
+
+register_part("mixer", "toy_ema", EmaMixer)
+register_part("feed_forward", "toy_routed", RoutedFeedForward)
+register_part("position", "toy_key_fade", KeyFade)
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyConfig(ModelConfig):
+    vocab_size: int
+    hidden_size: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    intermediate_size: int
+    window: int
+    decay: float
+    max_position_embeddings: int
+    eps: float = 1e-5
+
+
+def toy_spec(c: ToyConfig) -> ModelSpec:
+    H = c.hidden_size
+    norm = lambda name: PartSpec("rms_norm", {"size": H, "eps": c.eps}, {"weight": name})
+
+    def attn(i, window, position, qk_eps):
+        p = f"blocks.{i}.attn."
+        t = {"q_proj": p + "q", "k_proj": p + "k", "v_proj": p + "v", "o_proj": p + "o"}
+        if qk_eps is not None:
+            t.update(q_norm=p + "qn", k_norm=p + "kn")
+        return PartSpec("attention", {"hidden_size": H, "num_heads": c.heads, "num_kv_heads": c.kv_heads,
+                                      "head_dim": c.head_dim, "scale": None, "window": window,
+                                      "qk_norm_eps": qk_eps, "position": position}, t)
+
+    def mlp(i):
+        p = f"blocks.{i}.mlp."
+        return PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c.intermediate_size},
+                        {"gate_proj": p + "g", "up_proj": p + "u", "down_proj": p + "d"})
+
+    routed = PartSpec("toy_routed", {"hidden_size": H, "intermediate_size": c.intermediate_size, "experts": 2},
+                      dict([("router", "blocks.1.ffn.router")] +
+                           [(f"w{k}_{e}", f"blocks.1.ffn.w{k}_{e}") for k in (1, 2) for e in (0, 1)]))
+    blocks = [
+        BlockSpec(attn(0, None, "rotary", c.eps), mlp(0), norm("blocks.0.n1"), norm("blocks.0.n2")),
+        BlockSpec(PartSpec("toy_ema", {"hidden_size": H, "decay": c.decay}, {"w": "blocks.1.ema.w"}), routed,
+                  norm("blocks.1.n1"), norm("blocks.1.n2")),
+        BlockSpec(attn(2, c.window, "fade", None), mlp(2), norm("blocks.2.n1"), norm("blocks.2.n2")),
+        BlockSpec(attn(3, None, "rotary", c.eps), mlp(3), norm("blocks.3.n1"), norm("blocks.3.n2")),
+    ]
+    schedule = [LayerCall(0, cache=0), LayerCall(1, cache=1), LayerCall(2, cache=2),
+                LayerCall(0, cache=3),                           # block 0 a second time, a cache of its own
+                LayerCall(3, cache=0, writes_cache=False)]       # block 3 reads what the first call wrote
+    return ModelSpec(
+        architecture=c.architecture, hidden_size=H, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
+        embedding=PartSpec("token_embedding", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "embed"}),
+        positions={"rotary": PartSpec("rotary", {"head_dim": c.head_dim, "rotary_dim": c.head_dim // 2,
+                                                 "theta": 500.0, "max_position": c.max_position_embeddings}),
+                   "fade": PartSpec("toy_key_fade", {"horizon": 40.0})},
+        blocks=blocks, schedule=schedule, final_norm=norm("final_norm"),
+        head=PartSpec("linear_head", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "head"}))
+
+
+register_architecture("ToyForTests", ToyConfig, toy_spec)
+
+TOY = dict(architectures=["ToyForTests"], vocab_size=97, hidden_size=48, heads=4, kv_heads=2, head_dim=16,
+           intermediate_size=40, window=9, decay=0.8, max_position_embeddings=128, eps=1e-5)
+
+
+# ------------------------------------------------------------------ dense whole-sequence evaluation
+def toy_plain_logits(c, w, tokens):
+    T, D = len(tokens), c.head_dim
+    pos = torch.arange(T)
+    h = w["embed"][torch.tensor(tokens)]
+    kv0 = {}
+
+    def attention(x, i, window, kind, qk_eps, keep=None, reuse=None):
+        p = f"blocks.{i}.attn."
+        q = (x @ w[p + "q"].T).view(T, -1, D)
+        k = (x @ w[p + "k"].T).view(T, -1, D)
+        v = (x @ w[p + "v"].T).view(T, -1, D)
+        if qk_eps is not None:
+            q, k = plain.rms_norm(q, w[p + "qn"], qk_eps), plain.rms_norm(k, w[p + "kn"], qk_eps)
+        if kind == "rotary":
+            cos, sin = plain.rope_angles(pos, D // 2, 500.0)
+            q, k = plain.rope_rotate(q, cos, sin), plain.rope_rotate(k, cos, sin)
+        else:
+            k = k * (1.0 / (1.0 + pos.float() / 40.0))[:, None, None]
+        if keep is not None:
+            kv0[keep] = (k, v)
+        if reuse is not None:
+            k, v = kv0[reuse]
+        o = plain.causal_attention(q, k, v, pos, pos, D ** -0.5, window)
+        return o.reshape(T, -1) @ w[p + "o"].T
+
+    def swiglu(x, i):
+        p = f"blocks.{i}.mlp."
+        g = x @ w[p + "g"].T
+        return (g * torch.sigmoid(g) * (x @ w[p + "u"].T)) @ w[p + "d"].T
+
+    def block0(h, keep):
+        h = h + attention(plain.rms_norm(h, w["blocks.0.n1"], c.eps), 0, None, "rotary", c.eps, keep=keep)
+        return h + swiglu(plain.rms_norm(h, w["blocks.0.n2"], c.eps), 0)
+
+    h = block0(h, "first")
+    x = plain.rms_norm(h, w["blocks.1.n1"], c.eps)
+    u, s, ys = x @ w["blocks.1.ema.w"].T, torch.zeros(c.hidden_size), []
+    for t in range(T):
+        s = c.decay * s + u[t]
+        ys.append(s)
+    h = h + torch.stack(ys)
+    x = plain.rms_norm(h, w["blocks.1.n2"], c.eps)
+    choice = (x @ w["blocks.1.ffn.router"].T).argmax(-1)
+    y = torch.zeros_like(x)
+    for e in (0, 1):
+        m = choice == e
+        y[m] = (x[m] @ w[f"blocks.1.ffn.w1_{e}"].T).relu() @ w[f"blocks.1.ffn.w2_{e}"].T
+    h = h + y
+    h = h + attention(plain.rms_norm(h, w["blocks.2.n1"], c.eps), 2, c.window, "fade", None)
+    h = h + swiglu(plain.rms_norm(h, w["blocks.2.n2"], c.eps), 2)
+    h = block0(h, None)
+    h = h + attention(plain.rms_norm(h, w["blocks.3.n1"], c.eps), 3, None, "rotary", c.eps, reuse="first")
+    h = h + swiglu(plain.rms_norm(h, w["blocks.3.n2"], c.eps), 3)
+    return plain.rms_norm(h, w["final_norm"], c.eps) @ w["head"].T
+
+
+def run_toy(device, ops):
+    cfg = ToyConfig.from_dict(TOY)
+    spec = toy_spec(cfg)
+    weights = random_weights(spec, seed=4, std=0.08, norm_jitter=0.05, dtype="float32")
+    reqs = {rid: tt.random_tokens(cfg.vocab_size, n, seed=ord(rid)) for rid, n in
+            {"a": 40, "b": 7, "c": 23, "d": 61, "e": 1}.items()}
+    want = {rid: toy_plain_logits(cfg, weights, toks) for rid, toks in reqs.items()}
+    for cut in (tt.whole, tt.portions, tt.mixed):
+        steps = cut(reqs)
+        ec = EngineConfig(dtype="float32", page_size=4, max_token=tt.peak_tokens(steps), max_reside=4,
+                          max_step_tokens=256, prefill_chunk=256, device=device)
+        runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()},
+                             engine_config=ec, ops=ops)
+        cache = runner.cache
+        assert len(cache.groups) == 2 and len(cache.state_layers) == 1      # full, windowed; one state layer
+        got = tt.run_in_process(runner, steps)
+        for rid, toks in reqs.items():
+            for p in range(len(toks)):
+                torch.testing.assert_close(got[(rid, p)], want[rid][p], atol=3e-4, rtol=3e-4,
+                                           msg=lambda m: f"{cut.__name__} request {rid} position {p}: {m}")
+        windowed = [g for g in cache.groups if g.spec.window][0]
+        assert all(g.pages.in_use() == 0 for g in cache.groups) and windowed.spec.window == 9
+
+
+def test_toy_architecture_on_cpu_stand_in():
+    from tests.torch_ops import TorchOps
+    run_toy("cpu", TorchOps())
+
+
+@pytest.mark.gpu
+def test_toy_architecture_on_gpu():
+    run_toy("cuda:0", None)
