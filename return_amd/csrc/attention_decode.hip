@@ -150,8 +150,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
         }
 
         // ---- scores
-        float s[4][4];
-        float mx = -INFINITY;
+        float4_t cs[4];
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             float4_t c = {0.f, 0.f, 0.f, 0.f};
@@ -160,11 +159,18 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
                 c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[st][j], bq[j], c, 0, 0, 0);
             if constexpr (TAIL16)
                 c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak_tail[st], bq_tail, c, 0, 0, 0);
+            cs[st] = c;
+        }
+        MFMA_SETTLE();
+        float s[4][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int kp_abs = c0 + st * 16 + 4 * g + i;
                 const bool ok = kp_abs >= rg.lo && kp_abs <= rg.hi;
-                s[st][i] = ok ? c[i] * scale : -INFINITY;
+                s[st][i] = ok ? cs[st][i] * scale : -INFINITY;
                 mx = fmaxf(mx, s[st][i]);
             }
         }

@@ -1,0 +1,280 @@
+// Prefill attention for bfloat16: portions of prompts (two or more new tokens of a request)
+// over everything the paged cache holds for it, causal by position, optional window.
+//
+// What it restates of the reference: rollout/attention.py:45-142 (_prefill_kernel: packed
+// varlen causal GQA attention over paged K/V with online softmax; programs are (q tile,
+// segment, head); pages above the tile's last position are skipped, 103-106; mask
+// pos_q >= pos_k, 126-127). Different here: keys are already rotated in the cache; the grid
+// is a flat list of (request, q tile) made on the host instead of ceil(S/128) programs per
+// segment that mostly exit early (attention.py:168-174).
+//
+// BUILD-VARIANTS: PRE_PART=0 PRE_PART=1 PRE_PART=2 PRE_PART=3 PRE_API=1
+//
+// One workgroup of four waves per (q tile of 64 rows, query head); wave w owns rows 16w..16w+15.
+// Per pass a tile of BN keys is staged in LDS: K row-major (padded rows), V transposed.
+//  scores  S^T = K Q^T by MFMA 16x16x32 bf16: A = K tile rows from LDS, B = the wave's 16
+//          query rows held in registers. Lane (n, g) gets query n, keys 4g..4g+3 of each
+//          16-key tile.
+//  P.V     O^T += V^T P^T by the same MFMA. The contraction runs over keys in the order the
+//          lanes already hold them: k-slot (g, e) of a 32-key block is key 16*(e/4) + 4g + e%4,
+//          so P goes from the softmax registers straight into the B operand, and the A
+//          operand is two 8-byte reads of the transposed V tile.
+// A trailing 16 of D is a 16x16x32 step with the upper k half zero (one MFMA shape per chain).
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+#define PRE_BM 64
+
+#ifdef PRE_PART
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    return (uint32_t)f2bf_bits(a) | ((uint32_t)f2bf_bits(b) << 16);
+}
+
+union PK8 {
+    bf16x8_t v;
+    uint32_t w[4];
+    uint2 h[2];
+};
+
+template <int D16>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* __restrict__ k_pool,
+    const bf16* __restrict__ v_pool, const int* __restrict__ page_table,
+    const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
+    const int* __restrict__ cu_q, const int* __restrict__ q_start,
+    const int* __restrict__ tiles,       // [n_tiles][2]: request number, first row of the tile within it
+    int Hq, int Hkv, int P, float scale, int window) {
+    constexpr int D = 16 * D16;
+    constexpr int D32 = D / 32;
+    constexpr bool TAIL16 = (D % 32) != 0;
+    constexpr int BN = (D <= 128) ? 64 : 32;            // keys per pass
+    constexpr int KS = D + 8;                           // K tile row stride (elements): 16 bytes of padding
+    constexpr int VS = BN + 2;                          // V^T tile row stride (elements)
+    constexpr int LPR = D / 8;                          // threads that load one row (16 bytes each)
+
+    __shared__ __attribute__((aligned(16))) uint16_t k_s[BN * KS];
+    __shared__ __attribute__((aligned(16))) uint16_t vt_s[D * VS];
+    __shared__ int row_s[BN];
+
+    const int tile = blockIdx.x, head = blockIdx.y;
+    const int seg = tiles[2 * tile], q_off = tiles[2 * tile + 1];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int kvh = head / (Hq / Hkv);
+    const int q_len = cu_q[seg + 1] - cu_q[seg];
+    const int pos0 = q_start[seg];                       // position of the request's first new token
+    const int start = kv_start[seg];
+    const int* pt = page_table + cu_pages[seg];
+
+    // this lane's query row (for the B operand and for the mask): row n of the wave's 16
+    const int q_local = q_off + wave * 16 + n;
+    const bool q_ok = q_local < q_len;
+    const int pos_q = pos0 + q_local;
+    const bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8_t bq[D32 > 0 ? D32 : 1];
+    bf16x8_t bq_tail = z8;
+    {
+        const bf16* qp = q + ((size_t)(cu_q[seg] + (q_ok ? q_local : 0)) * Hq + head) * D;
+#pragma unroll
+        for (int j = 0; j < D32; ++j) {
+            bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(qp + 32 * j + 8 * g);
+            bq[j] = q_ok ? v : z8;
+        }
+        if constexpr (TAIL16) {
+            if (q_ok && g < 2) bq_tail = *reinterpret_cast<const bf16x8_t*>(qp + (D - 16) + 8 * g);
+        }
+    }
+
+    // keys this tile needs: from the earliest key any of its rows may read to its last row's position
+    const int tile_first_pos = pos0 + q_off;
+    const int tile_last_pos = pos0 + min(q_off + PRE_BM, q_len) - 1;
+    int first_key = start;
+    if (window > 0 && tile_first_pos - window + 1 > first_key) first_key = tile_first_pos - window + 1;
+
+    float m_run = -INFINITY, l_run = 0.f;
+    float4_t acc[D16];
+#pragma unroll
+    for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int c0 = (first_key / BN) * BN; c0 <= tile_last_pos; c0 += BN) {
+        // ---- stage the key tile: rows, then K row-major and V transposed
+        if (tid < BN) {
+            const int kpos = min(max(c0 + tid, first_key), tile_last_pos);
+            const int idx = kpos - start;
+            row_s[tid] = pt[idx / P] * P + idx % P;
+        }
+        __syncthreads();
+        for (int e = tid; e < BN * LPR; e += 256) {
+            const int key = e / LPR, c8 = (e % LPR) * 8;
+            const size_t src = ((size_t)row_s[key] * Hkv + kvh) * D + c8;
+            const uint4 kk = *reinterpret_cast<const uint4*>(k_pool + src);
+            *reinterpret_cast<uint4*>(&k_s[key * KS + c8]) = kk;
+            const uint4 vv = *reinterpret_cast<const uint4*>(v_pool + src);
+            const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                vt_s[(c8 + 2 * i) * VS + key] = (uint16_t)(w[i] & 0xffffu);
+                vt_s[(c8 + 2 * i + 1) * VS + key] = (uint16_t)(w[i] >> 16);
+            }
+        }
+        __syncthreads();
+
+        // ---- scores of the wave's 16 rows against the BN keys
+        float4_t cs[BN / 16];
+#pragma unroll
+        for (int st = 0; st < BN / 16; ++st) {
+            float4_t c = {0.f, 0.f, 0.f, 0.f};
+            const uint16_t* kr = &k_s[(st * 16 + n) * KS];
+#pragma unroll
+            for (int j = 0; j < D32; ++j) {
+                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(kr + 32 * j + 8 * g);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[j], c, 0, 0, 0);
+            }
+            if constexpr (TAIL16) {
+                bf16x8_t a = z8;
+                if (g < 2) a = *reinterpret_cast<const bf16x8_t*>(kr + (D - 16) + 8 * g);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq_tail, c, 0, 0, 0);
+            }
+            cs[st] = c;
+        }
+        MFMA_SETTLE();
+        float s[BN / 16][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int st = 0; st < BN / 16; ++st) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int kpos = c0 + st * 16 + 4 * g + i;
+                bool ok = kpos >= first_key && kpos <= pos_q;
+                if (window > 0) ok = ok && kpos > pos_q - window;
+                s[st][i] = ok ? cs[st][i] * scale : -INFINITY;
+                mx = fmaxf(mx, s[st][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        // a row that sees no key yet (all of this pass lies above it or outside its window) keeps m = -inf
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        float lsum = 0.f;
+#pragma unroll
+        for (int st = 0; st < BN / 16; ++st)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s[st][i] = (s[st][i] == -INFINITY) ? 0.f : __expf(s[st][i] - m_use);
+                lsum += s[st][i];
+            }
+        lsum += __shfl_xor(lsum, 16, 64);
+        lsum += __shfl_xor(lsum, 32, 64);
+        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_use);
+        l_run = l_run * alpha + lsum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < D16; ++dt) {
+            acc[dt][0] *= alpha;
+            acc[dt][1] *= alpha;
+            acc[dt][2] *= alpha;
+            acc[dt][3] *= alpha;
+        }
+
+        // ---- O^T += V^T P^T, 32 keys per MFMA
+#pragma unroll
+        for (int b = 0; b < BN / 32; ++b) {
+            PK8 pb;
+            pb.w[0] = pack2(s[2 * b][0], s[2 * b][1]);
+            pb.w[1] = pack2(s[2 * b][2], s[2 * b][3]);
+            pb.w[2] = pack2(s[2 * b + 1][0], s[2 * b + 1][1]);
+            pb.w[3] = pack2(s[2 * b + 1][2], s[2 * b + 1][3]);
+#pragma unroll
+            for (int dt = 0; dt < D16; ++dt) {
+                const uint16_t* vr = &vt_s[(dt * 16 + n) * VS + 32 * b + 4 * g];
+                PK8 va;
+                va.w[0] = *reinterpret_cast<const uint32_t*>(vr);
+                va.w[1] = *reinterpret_cast<const uint32_t*>(vr + 2);
+                va.w[2] = *reinterpret_cast<const uint32_t*>(vr + 16);
+                va.w[3] = *reinterpret_cast<const uint32_t*>(vr + 18);
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, acc[dt], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    MFMA_SETTLE();
+    // ---- acc[dt][i] = O^T[d = 16dt + 4g + i][query n]
+    if (q_ok) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        bf16* op = out + ((size_t)(cu_q[seg] + q_local) * Hq + head) * D;
+#pragma unroll
+        for (int dt = 0; dt < D16; ++dt) {
+            uint2 w;
+            w.x = pack2(acc[dt][0] * inv, acc[dt][1] * inv);
+            w.y = pack2(acc[dt][2] * inv, acc[dt][3] * inv);
+            *reinterpret_cast<uint2*>(op + dt * 16 + 4 * g) = w;
+        }
+    }
+}
+
+#define PRE_CAT2(a, b) a##b
+#define PRE_CAT(a, b) PRE_CAT2(a, b)
+// head sizes 16*(4*PRE_PART+1) .. 16*(4*PRE_PART+4)
+extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, dim3 grid, hipStream_t st, const bf16* q, bf16* out,
+                                              const bf16* kp, const bf16* vp, const int* pt,
+                                              const int* cup, const int* kvs, const int* cuq,
+                                              const int* qs, const int* tiles, int Hq, int Hkv, int P,
+                                              float scale, int window) {
+#define PRE_CASE(N)                                                                               \
+    case N:                                                                                       \
+        hipLaunchKernelGGL(attn_prefill_kernel<N>, grid, dim3(256), 0, st, q, out, kp, vp, pt, cup, \
+                           kvs, cuq, qs, tiles, Hq, Hkv, P, scale, window);                       \
+        return RA_OK;
+    switch (D16) {
+        PRE_CASE(4 * PRE_PART + 1) PRE_CASE(4 * PRE_PART + 2) PRE_CASE(4 * PRE_PART + 3)
+        PRE_CASE(4 * PRE_PART + 4)
+        default: return RA_ERR_ARG;
+    }
+#undef PRE_CASE
+}
+#endif  // PRE_PART
+
+#ifdef PRE_API
+#define PRE_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
+    const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs,    \
+    const int* tiles, int Hq, int Hkv, int P, float scale, int window
+extern "C" int ra_pre_part_0(PRE_PART_ARGS);
+extern "C" int ra_pre_part_1(PRE_PART_ARGS);
+extern "C" int ra_pre_part_2(PRE_PART_ARGS);
+extern "C" int ra_pre_part_3(PRE_PART_ARGS);
+
+// tiles: int32 [n_tiles][2] = (request number, first row of the tile within the request's new
+// tokens); every request with more than one new token is covered in tiles of 64 rows.
+extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k_pool,
+                                         const void* v_pool, const int* page_table,
+                                         const int* cu_pages, const int* kv_start, const int* cu_q,
+                                         const int* q_start, const int* tiles, int n_tiles, int Hq,
+                                         int Hkv, int D, int P, float scale, int window, void* stream) {
+    if (n_tiles <= 0) return RA_OK;
+    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || Hq > 65535 || P <= 0)
+        return RA_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(n_tiles, Hq);
+    const int d16 = D / 16;
+    int rc;
+#define GO(k)                                                                                      \
+    rc = ra_pre_part_##k(d16, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
+                         (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tiles, \
+                         Hq, Hkv, P, scale, window)
+    switch ((d16 - 1) / 4) {
+        case 0: GO(0); break;
+        case 1: GO(1); break;
+        case 2: GO(2); break;
+        case 3: GO(3); break;
+        default: return RA_ERR_ARG;
+    }
+#undef GO
+    if (rc != RA_OK) return rc;
+    return ra_launch_status();
+}
+#endif  // PRE_API

@@ -73,5 +73,16 @@ static inline int ra_launch_status() {
     return hipGetLastError() == hipSuccess ? RA_OK : RA_ERR_LAUNCH;
 }
 
+// Placed between the last MFMA of a chain and the first read of its result. hipcc inserts
+// the wait states an MFMA result needs only when producer and reader sit in one basic block;
+// with a branch in between (a mask, a loop exit) the 16x16x32 bf16 result was read too early
+// on gfx950 and its last register still held the previous value. Nothing is scheduled across.
+#define MFMA_SETTLE()                        \
+    do {                                     \
+        __builtin_amdgcn_sched_barrier(0);   \
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7" ::: "memory"); \
+        __builtin_amdgcn_sched_barrier(0);   \
+    } while (0)
+
 #define RA_DTYPE_F32 0
 #define RA_DTYPE_BF16 1

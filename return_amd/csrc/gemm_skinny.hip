@@ -60,6 +60,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
                 for (int b = 0; b < MB; ++b)
                     c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bx[b][u], c[b], 0, 0, 0);
         }
+        MFMA_SETTLE();
         // c[b][i] = partial y[m = 16b + n][row n0 + 4g + i]
 #pragma unroll
         for (int b = 0; b < MB; ++b)

@@ -62,6 +62,7 @@ def _declare(lib):
         "ra_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
+        "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
     }
     for name, args in sigs.items():
@@ -315,6 +316,13 @@ class HipOps:
             toks, n_tok = step.prefill_toks, step.n_prefill_tokens
         else:
             toks, n_tok = None, T
+        if q.dtype == torch.bfloat16 and step.n_prefill_tiles > 0 and D % 16 == 0 and D <= 256 and \
+                (fast_decode or step.n_decode == 0):
+            self._check(self.lib.ra_attention_prefill_bf16(
+                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(step.prefill_tiles),
+                step.n_prefill_tiles, n_q, n_kv, D, P, float(scale), window, self._stream()),
+                "attention_prefill_bf16")
+            return
         self._check(self.lib.ra_attention_plain(
             _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
             n_q, n_kv, D, P, float(scale), window, _code(q.dtype), self._stream()), "attention_plain")

@@ -204,6 +204,9 @@ def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
                  n_prefill_tokens=cu_q[-1] - len(dec),
                  prefill_toks=i32([t for i in pre for t in range(cu_q[i], cu_q[i + 1])]) if both else None,
                  prefill_segs=pre)
+    from return_amd.engine.batch import prefill_tiles
+    tiles = prefill_tiles(q_lens)
+    extra.update(n_prefill_tiles=len(tiles), prefill_tiles=i32(tiles) if tiles else None)
     return types.SimpleNamespace(**extra, n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
                                  seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
                                  q_lens=list(q_lens), q_starts=list(q_starts),
@@ -251,6 +254,28 @@ def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
     ops.attention(q, a, kp, vp, step, 0, D ** -0.5, window)
     ref.attention(q, b, kp, vp, step, 0, D ** -0.5, window)
     torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("D", list(range(16, 257, 16)))
+def test_prefill_attention_every_head_size(ops, ref, D):
+    """The bfloat16 prefill kernel at every head size it takes: whole prompts, portions with
+    context, tiles that end inside a page, a window."""
+    for (Hq, Hkv), window in (((4, 2), 0), ((3, 1), 37)):
+        P = 16
+        segs = [(70, 0), (2, 131), (65, 64), (5, 3)]
+        need = [-(-(a + b) // P) for a, b in segs]
+        pages_of, nxt = [], 0
+        for k in need:
+            pages_of.append(list(range(nxt, nxt + k)))
+            nxt += k
+        step = _step([s[0] for s in segs], [s[1] for s in segs], P, pages_of)
+        kp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D)
+        vp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D + 1)
+        q = rnd(sum(s[0] for s in segs), Hq, D, dtype=torch.bfloat16, seed=D + 2)
+        a, b = torch.zeros_like(q), torch.zeros_like(q)
+        ops.attention(q, a, kp, vp, step, 0, D ** -0.5, window)
+        ref.attention(q, b, kp, vp, step, 0, D ** -0.5, window)
+        torch.testing.assert_close(a.float(), b.float(), **tol(torch.bfloat16))
 
 
 @pytest.mark.parametrize("D", list(range(16, 257, 16)))
