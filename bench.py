@@ -38,7 +38,7 @@ PAGE = 16
 PREFILL_TOKENS = 2048
 
 
-def build_runner(layers, dtype, max_reside, seed=0):
+def build_runner(layers, dtype, max_reside, seed=0, use_graphs=True):
     import torch
     import return_amd.models  # noqa: F401
     from return_amd.config import EngineConfig, Qwen3Config
@@ -53,7 +53,7 @@ def build_runner(layers, dtype, max_reside, seed=0):
                              generator_device="cuda:0")
     ec = EngineConfig(dtype=dtype, page_size=PAGE, max_token=max_reside * MAX_CONTEXT,
                       max_reside=max_reside, max_step_tokens=max(PREFILL_TOKENS, max_reside),
-                      prefill_chunk=PREFILL_TOKENS)
+                      prefill_chunk=PREFILL_TOKENS, use_graphs=use_graphs)
     runner = ModelRunner(config=cfg, weights=weights, engine_config=ec)
     del weights
     torch.cuda.empty_cache()
@@ -103,8 +103,7 @@ def decode_steps(runner, ids, steps, warmup, vocab):
 
     def one():
         nonlocal toks
-        logits = runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)])
-        toks, _ = runner.sample(logits, zeros, [0] * n, ones, zeros)
+        toks, _, _ = runner.decode_and_sample(ids, toks, zeros, [0] * n, ones, zeros)
 
     for _ in range(warmup):
         one()
@@ -130,6 +129,7 @@ def main():
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--no-graphs", action="store_true", help="launch every kernel from the host instead of replaying HIP graphs")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -140,7 +140,8 @@ def main():
         print("bench.py: no GPU visible")
         return 1
     elt = 2 if args.dtype == "bfloat16" else 4
-    cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch))
+    cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),
+                               use_graphs=not args.no_graphs)
     V = cfg.vocab_size
 
     # ---- headline: decode at the given batch
@@ -190,6 +191,7 @@ def main():
                    "intermediate": cfg.intermediate_size, "vocab": V, "global_batch": args.batch,
                    "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": PAGE,
                    "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
+                   "hip_graphs": not args.no_graphs,
                    "weights": "random N(0,0.02)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},

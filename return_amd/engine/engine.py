@@ -81,11 +81,21 @@ class Engine:
         if not plan.entries:
             return ended
         t0 = time.perf_counter()
-        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
-                   for e in plan.entries]
-        logits = self.runner.step(entries)
         sampled: Dict[object, tuple] = {}
         rows = [e.request for e in plan.entries if e.sample]
+        if len(rows) == len(plan.entries) and all(len(e.tokens) == 1 for e in plan.entries):
+            # decode only: one call that runs the model and the sampler (from a graph if enabled)
+            toks, logps, _ = self.runner.decode_and_sample(
+                [r.id for r in rows], [e.tokens[0] for e in plan.entries],
+                [r.params.temperature for r in rows], [r.params.top_k for r in rows],
+                [r.params.top_p for r in rows], [r.stream.next() for r in rows])
+            for r, t, lp in zip(rows, toks, logps):
+                sampled[r.id] = (t, lp)
+            rows = []
+        else:
+            entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
+                       for e in plan.entries]
+            logits = self.runner.step(entries)
         if rows:
             toks, logps = self.runner.sample(
                 logits, [r.params.temperature for r in rows], [r.params.top_k for r in rows],

@@ -61,6 +61,16 @@ class ModelRunner:
         self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device)
         self.vocab_size = self.spec.vocab_size
         self.max_position = self.spec.max_position
+        # decode-only steps replayed from captured HIP graphs (rollout/model.py:346-407 captures one
+        # graph per batch size; here one per (batch size, context bucket))
+        self._graphs = {}
+        self._graph_pool = None
+        n = ec.max_reside
+        pin = self.rt.device.type == "cuda"
+        self._samp_host_f = torch.zeros(3, n, dtype=torch.float32, pin_memory=pin)
+        self._samp_host_k = torch.zeros(n, dtype=torch.int32, pin_memory=pin)
+        self._samp_dev_f = torch.zeros(3, n, dtype=torch.float32, device=self.rt.device)
+        self._samp_dev_k = torch.zeros(n, dtype=torch.int32, device=self.rt.device)
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request_id) -> None:
@@ -107,6 +117,83 @@ class ModelRunner:
         finally:
             self.cache.end_step()
         return logits
+
+    # ------------------------------------------------------------------ decode from a graph
+    def _put_sampling(self, m, temperature, top_k, top_p, uniforms):
+        self._samp_host_f[0, :m] = torch.as_tensor(temperature, dtype=torch.float32)
+        self._samp_host_f[1, :m] = torch.as_tensor(top_p, dtype=torch.float32)
+        self._samp_host_f[2, :m] = torch.as_tensor(uniforms, dtype=torch.float32)
+        self._samp_host_k[:m] = torch.as_tensor(top_k, dtype=torch.int32)
+        self._samp_dev_f.copy_(self._samp_host_f, non_blocking=True)
+        self._samp_dev_k.copy_(self._samp_host_k, non_blocking=True)
+
+    def _decode_body(self, batch):
+        logits = self.model.forward(batch, self.cache)
+        m = batch.n_logit_rows
+        picked = self.rt.ops.sample(logits, self._samp_dev_f[0, :m], self._samp_dev_k[:m],
+                                    self._samp_dev_f[1, :m], self._samp_dev_f[2, :m])
+        return logits, picked
+
+    def decode_and_sample(self, request_ids, tokens, temperature, top_k, top_p, uniforms):
+        """One token per request, logits sampled at once: the steady state of generation.
+
+        With use_graphs the whole step (model and sampler) is one captured HIP graph per
+        (batch size, context bucket); tables and sampling options go into fixed buffers first.
+        Returns (tokens, logprobs, logits); logits stay on the device.
+        """
+        n = len(request_ids)
+        for rid, t in zip(request_ids, tokens):
+            if not 0 <= int(t) < self.vocab_size:
+                raise ValueError(f"request {rid!r}: token {t} outside the vocabulary of {self.vocab_size}")
+            if self.cache.seq_len(rid) + 1 > self.max_position:
+                raise ValueError(f"request {rid!r} would pass max_position_embeddings {self.max_position}")
+        tables = self.cache.begin_step([(rid, 1) for rid in request_ids])
+        try:
+            batch = self.builder.build(tables, [[int(t)] for t in tokens], list(range(n)))
+            self._put_sampling(n, temperature, top_k, top_p, uniforms)
+            with torch.no_grad():
+                if self.engine_config.use_graphs and self.rt.device.type == "cuda":
+                    logits, picked = self._replay(batch)
+                else:
+                    logits, picked = self._decode_body(batch)
+        finally:
+            self.cache.end_step()
+        host = picked.cpu()
+        return host[:, 0].tolist(), host[:, 1].contiguous().view(torch.float32).tolist(), logits
+
+    def _replay(self, batch):
+        bucket = 256
+        while bucket < batch.max_decode_seq_len:
+            bucket *= 2
+        key = (batch.n_seqs, bucket)
+        entry = self._graphs.get(key)
+        batch.max_decode_seq_len = bucket        # grid and scratch sizes cover the whole bucket
+        if entry is None:
+            ops = self.rt.ops
+            saved = getattr(ops, "decode_split_tokens", None)
+            if saved is not None and saved <= 0:
+                # the split size is part of the captured launch: fix it from the bucket
+                chunks = batch.n_seqs * max(1, self.model.max_kv_heads()) * (bucket // 64)
+                ops.decode_split_tokens = 64 * max(1, min(8, chunks // 4096))
+            split = getattr(ops, "decode_split_tokens", None)
+            side = torch.cuda.Stream(self.rt.device)
+            side.wait_stream(torch.cuda.current_stream(self.rt.device))
+            with torch.cuda.stream(side):
+                self._decode_body(batch)                      # warm-up outside the capture
+            torch.cuda.current_stream(self.rt.device).wait_stream(side)
+            torch.cuda.synchronize(self.rt.device)
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits, picked = self._decode_body(batch)
+            if saved is not None:
+                ops.decode_split_tokens = saved
+            entry = (graph, logits, picked, split)
+            self._graphs[key] = entry
+        graph, logits, picked, _ = entry
+        graph.replay()
+        return logits, picked
 
     def sample(self, logits: torch.Tensor, temperature, top_k, top_p, uniforms):
         """Choose a token per logits row on the device; returns (tokens, logprobs) as Python lists."""

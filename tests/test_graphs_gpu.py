@@ -1,0 +1,61 @@
+"""Decode steps replayed from captured HIP graphs give what the eager path gives, on every
+replay, with eager work and synchronisations between the replays."""
+import pytest
+import torch
+
+from return_amd.config import EngineConfig
+from return_amd.engine import ModelRunner, StepEntry
+from tests import trace_tools as tt
+from tests.conftest import TINY_B
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_graph_replays_match_eager(folder_b, dtype):
+    V = TINY_B["vocab_size"]
+    prompts = {rid: tt.random_tokens(V, n, seed=n) for rid, n in {"a": 40, "b": 7, "c": 130}.items()}
+
+    def make(use_graphs):
+        ec = EngineConfig(dtype=dtype, page_size=16, max_token=4096, max_reside=4, max_step_tokens=512,
+                          prefill_chunk=512, use_graphs=use_graphs)
+        r = ModelRunner(folder_b, engine_config=ec)
+        for rid, toks in prompts.items():
+            r.add_request(rid)
+            r.step([StepEntry(rid, toks, [])])
+        return r
+
+    eager, graph = make(False), make(True)
+    ids = list(prompts)
+    toks_e = toks_g = [3, 5, 7]
+    temps, ks, ps = [0.0, 0.8, 0.0], [0, 5, 0], [1.0, 0.9, 1.0]
+    for step in range(140):                     # crosses pages and the 256-token context bucket
+        us = [0.1 * ((step * 7 + i) % 10) for i in range(3)]
+        te, le, logits_e = eager.decode_and_sample(ids, toks_e, temps, ks, ps, us)
+        tg, lg, logits_g = graph.decode_and_sample(ids, toks_g, temps, ks, ps, us)
+        assert torch.equal(logits_e, logits_g), f"replay {step} differs from the eager step"
+        assert te == tg and le == lg
+        toks_e = toks_g = te
+        if step % 9 == 0:                       # eager work of the program's own between replays
+            graph.add_request("x")
+            graph.step([StepEntry("x", tt.random_tokens(V, 20, seed=step), [19])])
+            graph.free_request("x")
+            torch.cuda.synchronize()
+    assert len(graph._graphs) >= 2              # more than one context bucket was captured
+    # a different batch size gets a graph of its own
+    graph.free_request("b"); eager.free_request("b")
+    te, _, logits_e = eager.decode_and_sample(["a", "c"], [1, 2], [0.0, 0.0], [0, 0], [1.0, 1.0], [0.0, 0.0])
+    tg, _, logits_g = graph.decode_and_sample(["a", "c"], [1, 2], [0.0, 0.0], [0, 0], [1.0, 1.0], [0.0, 0.0])
+    assert te == tg and torch.equal(logits_e, logits_g)
+
+
+def test_generation_with_graphs(folder_b):
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (1, 8, 31, 64, 100)]
+    outs = []
+    for use_graphs in (False, True):
+        eng = Engine(folder_b, dtype="float32", page_size=32, max_token=4096, max_reside=5,
+                     max_step_tokens=64, prefill_chunk=24, use_graphs=use_graphs)
+        outs.append([r.output_ids for r in eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=20))])
+    assert outs[0] == outs[1]
