@@ -60,15 +60,88 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
     }
 }
 
+// The same with 16-byte accesses and the row kept in registers between the two phases:
+// H % 4 == 0 and H <= 4 * VPT * blockDim. One block per output row.
+template <typename T, int VPT>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                       const float* __restrict__ w, float eps, T* __restrict__ out,
+                                       const int* __restrict__ rows, int H) {
+    __shared__ float scratch[16];
+    const int m = blockIdx.x;
+    const size_t r = rows ? (size_t)rows[m] : (size_t)m;
+    float4* hr = reinterpret_cast<float4*>(h + r * H);
+    const bool write_back = (rows == nullptr) && (delta != nullptr);
+    const int nv = H >> 2;
+    float4 v[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * blockDim.x;
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < nv) {
+            v[i] = hr[c];
+            if (delta) {
+                if constexpr (sizeof(T) == 2) {
+                    const uint2 d = *reinterpret_cast<const uint2*>(delta + r * H + 4 * c);
+                    v[i].x += __uint_as_float(d.x << 16);
+                    v[i].y += __uint_as_float(d.x & 0xffff0000u);
+                    v[i].z += __uint_as_float(d.y << 16);
+                    v[i].w += __uint_as_float(d.y & 0xffff0000u);
+                } else {
+                    const float4 d = *reinterpret_cast<const float4*>(delta + r * H + 4 * c);
+                    v[i].x += d.x; v[i].y += d.y; v[i].z += d.z; v[i].w += d.w;
+                }
+            }
+            if (write_back) hr[c] = v[i];
+            ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    T* o = out + (size_t)m * H;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * blockDim.x;
+        if (c < nv) {
+            const float4 ww = reinterpret_cast<const float4*>(w)[c];
+            const float a = v[i].x * rstd * ww.x, b = v[i].y * rstd * ww.y;
+            const float cc = v[i].z * rstd * ww.z, d = v[i].w * rstd * ww.w;
+            if constexpr (sizeof(T) == 2) {
+                uint2 p;
+                p.x = (uint32_t)f2bf_bits(a) | ((uint32_t)f2bf_bits(b) << 16);
+                p.y = (uint32_t)f2bf_bits(cc) | ((uint32_t)f2bf_bits(d) << 16);
+                *reinterpret_cast<uint2*>(o + 4 * c) = p;
+            } else {
+                *reinterpret_cast<float4*>(o + 4 * c) = make_float4(a, b, cc, d);
+            }
+        }
+    }
+}
+
 extern "C" int ra_add_rmsnorm(float* h, const void* delta, const float* w, float eps, void* out,
                               const int* rows, int M, int H, int dtype, void* stream) {
     if (M <= 0) return RA_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (H % 4 == 0 && H <= 16384) {
+        const int nv = H / 4;
+        const int threads = nv <= 256 ? 256 : (nv <= 512 ? 512 : 1024);
+        dim3 grid(M), block(threads);
+        const bool one = nv <= threads;              // one vector per thread, else up to four
+        if (dtype == RA_DTYPE_F32) {
+            if (one) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<float, 1>), grid, block, 0, st, h, (const float*)delta, w, eps, (float*)out, rows, H);
+            else hipLaunchKernelGGL((add_rmsnorm_vec_kernel<float, 4>), grid, block, 0, st, h, (const float*)delta, w, eps, (float*)out, rows, H);
+        } else {
+            if (one) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<bf16, 1>), grid, block, 0, st, h, (const bf16*)delta, w, eps, (bf16*)out, rows, H);
+            else hipLaunchKernelGGL((add_rmsnorm_vec_kernel<bf16, 4>), grid, block, 0, st, h, (const bf16*)delta, w, eps, (bf16*)out, rows, H);
+        }
+        return ra_launch_status();
+    }
     dim3 grid(M), block(H >= 2048 ? 512 : 256);
     if (dtype == RA_DTYPE_F32)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, (hipStream_t)stream, h,
+        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, st, h,
                            (const float*)delta, w, eps, (float*)out, rows, H);
     else
-        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, grid, block, 0, (hipStream_t)stream, h,
+        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, grid, block, 0, st, h,
                            (const bf16*)delta, w, eps, (bf16*)out, rows, H);
     return ra_launch_status();
 }

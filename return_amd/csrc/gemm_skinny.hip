@@ -9,6 +9,10 @@
 // distributed over lanes as long as both operands agree. Partial tiles of the waves are
 // added through LDS in wave order, so the result does not depend on scheduling.
 // Needs K % 8 == 0 (16-byte loads); other K go to the plain kernel.
+//
+// GATED: W is [2I, K] with the gate rows first (rollout/monkey_patch/qwen3.py:103); a tile
+// takes 16 gate rows and the 16 up rows that belong to them and writes silu(g) * u
+// (rollout/fused.py:103-114) as [M, I], so the [M, 2I] intermediate never reaches memory.
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -17,11 +21,13 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 #define SK_UNROLL 8                      // MFMA steps (of 32 k) per wave iteration
 #define SK_KB (32 * SK_UNROLL)           // k elements per wave iteration
 
-template <int WAVES, int MB, typename TO>
+template <int WAVES, int MB, typename TO, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ W, TO* __restrict__ out, int M, int N,
     int K, int n_tiles) {
-    __shared__ float red[WAVES][MB][16][17];
+    // N: rows of the result (= rows of W, or half of them when GATED)
+    constexpr int NG = GATED ? 2 : 1;
+    __shared__ float red[WAVES][NG][MB][16][17];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n = lane & 15, g = lane >> 4;
     const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -30,6 +36,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         const int n0 = tile * 16;
         const int row = min(n0 + n, N - 1);                 // clamped: loads stay inside W
         const bf16* wp = W + (size_t)row * K + g * 8;
+        const bf16* wp_up = wp + (size_t)N * K;               // GATED: the up row of the same column
         const bf16* xp[MB];
         bool x_ok[MB];
 #pragma unroll
@@ -38,18 +45,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
             x_ok[b] = m < M;
             xp[b] = x + (size_t)min(m, M - 1) * K + g * 8;
         }
-        float4_t c[MB];
+        float4_t c[NG][MB];
 #pragma unroll
-        for (int b = 0; b < MB; ++b) c[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int z = 0; z < NG; ++z)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) c[z][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
         for (int kb = wave * SK_KB; kb < K; kb += WAVES * SK_KB) {
-            bf16x8_t a[SK_UNROLL];
+            bf16x8_t a[NG][SK_UNROLL];
             bf16x8_t bx[MB][SK_UNROLL];
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u) {
                 const int k = kb + u * 32;
                 const bool in = k + g * 8 < K;               // K % 8 == 0: a lane's 8 are in or out together
-                a[u] = in ? *reinterpret_cast<const bf16x8_t*>(wp + k) : zero;
+                a[0][u] = in ? *reinterpret_cast<const bf16x8_t*>(wp + k) : zero;
+                if constexpr (GATED) a[1][u] = in ? *reinterpret_cast<const bf16x8_t*>(wp_up + k) : zero;
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
                     bx[b][u] = (in && x_ok[b]) ? *reinterpret_cast<const bf16x8_t*>(xp[b] + k) : zero;
@@ -58,14 +68,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
             for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
-                    c[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bx[b][u], c[b], 0, 0, 0);
+#pragma unroll
+                    for (int z = 0; z < NG; ++z)
+                        c[z][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[z][u], bx[b][u], c[z][b], 0, 0, 0);
         }
         MFMA_SETTLE();
-        // c[b][i] = partial y[m = 16b + n][row n0 + 4g + i]
+        // c[z][b][i] = partial y[m = 16b + n][row n0 + 4g + i]
 #pragma unroll
-        for (int b = 0; b < MB; ++b)
+        for (int z = 0; z < NG; ++z)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[wave][b][4 * g + i][n] = c[b][i];
+            for (int b = 0; b < MB; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[wave][z][b][4 * g + i][n] = c[z][b][i];
         __syncthreads();
         for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
             const int b = e >> 8, mm = (e >> 4) & 15, r = e & 15;     // r fastest: neighbours write neighbours
@@ -73,7 +87,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
             if (m < M && col < N) {
                 float s = 0.f;
 #pragma unroll
-                for (int w = 0; w < WAVES; ++w) s += red[w][b][r][mm];
+                for (int w = 0; w < WAVES; ++w) s += red[w][0][b][r][mm];
+                if constexpr (GATED) {
+                    float u = 0.f;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) u += red[w][1][b][r][mm];
+                    s = s / (1.0f + expf(-s)) * u;        // gate and up stay 32-bit until here
+                }
                 out[(size_t)m * N + col] = from_f<TO>(s);
             }
         }
@@ -81,21 +101,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     }
 }
 
-template <int WAVES, int MB, typename TO>
+template <int WAVES, int MB, typename TO, bool GATED>
 static void launch_skinny(int grid, hipStream_t st, const bf16* x, const bf16* W, TO* out, int M,
                           int N, int K, int n_tiles) {
-    hipLaunchKernelGGL((gemm_skinny_kernel<WAVES, MB, TO>), dim3(grid), dim3(WAVES * 64), 0, st, x,
-                       W, out, M, N, K, n_tiles);
+    hipLaunchKernelGGL((gemm_skinny_kernel<WAVES, MB, TO, GATED>), dim3(grid), dim3(WAVES * 64), 0,
+                       st, x, W, out, M, N, K, n_tiles);
 }
 
 template <int WAVES, typename TO>
 static int pick_mb(int grid, hipStream_t st, const bf16* x, const bf16* W, TO* out, int M, int N,
                    int K, int n_tiles) {
     switch ((M + 15) / 16) {
-        case 1: launch_skinny<WAVES, 1, TO>(grid, st, x, W, out, M, N, K, n_tiles); break;
-        case 2: launch_skinny<WAVES, 2, TO>(grid, st, x, W, out, M, N, K, n_tiles); break;
-        case 3: launch_skinny<WAVES, 3, TO>(grid, st, x, W, out, M, N, K, n_tiles); break;
-        case 4: launch_skinny<WAVES, 4, TO>(grid, st, x, W, out, M, N, K, n_tiles); break;
+        case 1: launch_skinny<WAVES, 1, TO, false>(grid, st, x, W, out, M, N, K, n_tiles); break;
+        case 2: launch_skinny<WAVES, 2, TO, false>(grid, st, x, W, out, M, N, K, n_tiles); break;
+        case 3: launch_skinny<WAVES, 3, TO, false>(grid, st, x, W, out, M, N, K, n_tiles); break;
+        case 4: launch_skinny<WAVES, 4, TO, false>(grid, st, x, W, out, M, N, K, n_tiles); break;
         default: return RA_ERR_ARG;
     }
     return RA_OK;
@@ -120,5 +140,19 @@ extern "C" int ra_gemm_skinny_bf16(const void* x, const void* W, void* out, int 
                                        : pick_mb<4, bf16>(grid, st, xx, ww, (bf16*)out, M, N, K, n_tiles);
     }
     if (rc != RA_OK) return rc;
+    return ra_launch_status();
+}
+
+// out [M, I] = silu(x @ Wg^T) * (x @ Wu^T) for W = [Wg; Wu] of shape [2I, K]; M <= 16.
+extern "C" int ra_gemm_skinny_gated_bf16(const void* x, const void* W, void* out, int M, int I, int K,
+                                         void* stream) {
+    if (M <= 0 || I <= 0) return RA_OK;
+    if (M > 16 || K <= 0 || K % 8 != 0) return RA_ERR_ARG;
+    const int n_tiles = (I + 15) / 16;
+    hipStream_t st = (hipStream_t)stream;
+    if (n_tiles <= 512)
+        launch_skinny<8, 1, bf16, true>(n_tiles, st, (const bf16*)x, (const bf16*)W, (bf16*)out, M, I, K, n_tiles);
+    else
+        launch_skinny<4, 1, bf16, true>(n_tiles, st, (const bf16*)x, (const bf16*)W, (bf16*)out, M, I, K, n_tiles);
     return ra_launch_status();
 }

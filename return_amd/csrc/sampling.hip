@@ -12,7 +12,7 @@
 // Tokens that tie with the k-th value, or with the top-p boundary value, are all kept.
 #include "common.h"
 
-#define SAMPLE_THREADS 256
+#define SAMPLE_THREADS 1024
 
 __device__ __forceinline__ uint32_t order_key(float f) {
     const uint32_t b = __float_as_uint(f);
@@ -31,24 +31,53 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* x = logits + (size_t)row * V;
 
-    // ---- raw maximum, first index that holds it, log-sum-exp
-    float mx = -INFINITY;
+    // ---- one pass: running maximum, first index that holds it, sum of exp(x - maximum)
+    float mx = -INFINITY, se = 0.f;
     int arg = 0x7fffffff;
-    for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const float v = x[i];
-        if (v > mx) { mx = v; arg = i; }
+    auto take = [&](float v, int i) {
+        if (v > mx) {
+            se = se * __expf(mx - v) + 1.0f;          // mx = -inf: se is 0 and stays finite
+            mx = v;
+            arg = i;
+        } else {
+            se += __expf(v - mx);
+        }
+    };
+    if ((V & 3) == 0) {
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+        for (int i = tid; i < (V >> 2); i += SAMPLE_THREADS) {
+            const float4 v = x4[i];
+            take(v.x, 4 * i); take(v.y, 4 * i + 1); take(v.z, 4 * i + 2); take(v.w, 4 * i + 3);
+        }
+    } else {
+        for (int i = tid; i < V; i += SAMPLE_THREADS) take(x[i], i);
     }
-    const float gmax = block_max(mx, scratch);
+    // merge (mx, se, arg) over the wave, then over the waves in wave order
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float m2 = __shfl_xor(mx, o, 64), s2 = __shfl_xor(se, o, 64);
+        const int a2 = __shfl_xor(arg, o, 64);
+        const float m = fmaxf(mx, m2);
+        const float s1 = (mx == -INFINITY) ? 0.f : se * __expf(mx - m);
+        const float s3 = (m2 == -INFINITY) ? 0.f : s2 * __expf(m2 - m);
+        arg = (m2 > mx) ? a2 : ((m2 == mx) ? min(arg, a2) : arg);
+        se = s1 + s3;                                 // the same two numbers in both lanes of a pair
+        mx = m;
+    }
+    __shared__ float wm[16], ws[16];
+    __shared__ int wa[16];
+    if ((tid & 63) == 0) { wm[tid >> 6] = mx; ws[tid >> 6] = se; wa[tid >> 6] = arg; }
     __syncthreads();
-    if (tid == 0) sh_int[0] = 0x7fffffff;
-    __syncthreads();
-    if (mx == gmax) atomicMin(&sh_int[0], arg);
-    __syncthreads();
-    const int argmax = sh_int[0];
-    float se = 0.f;
-    for (int i = tid; i < V; i += SAMPLE_THREADS) se += expf(x[i] - gmax);
-    se = block_sum(se, scratch);
-    const float lse = gmax + logf(se);
+    float gmax = wm[0];
+    int argmax = wa[0];
+    for (int w = 1; w < SAMPLE_THREADS / 64; ++w) {
+        if (wm[w] > gmax) { gmax = wm[w]; argmax = wa[w]; }
+        else if (wm[w] == gmax) argmax = min(argmax, wa[w]);
+    }
+    float tot = 0.f;
+    for (int w = 0; w < SAMPLE_THREADS / 64; ++w)
+        tot += (wm[w] == -INFINITY) ? 0.f : ws[w] * __expf(wm[w] - gmax);
+    const float lse = gmax + logf(tot);
 
     const float temp = temperature[row];
     if (!(temp > 0.f)) {
@@ -67,7 +96,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         uint32_t prefix = 0u, mask = 0u;
         int remaining = k;
         for (int shift = 24; shift >= 0; shift -= 8) {
-            hist[tid] = 0;
+            if (tid < 256) hist[tid] = 0;
             __syncthreads();
             for (int i = tid; i < V; i += SAMPLE_THREADS) {
                 const uint32_t key = order_key(x[i]);

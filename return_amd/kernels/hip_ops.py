@@ -60,6 +60,7 @@ def _declare(lib):
         "ra_silu_mul": [P, P, I, I, I, P],
         "ra_gemm_nt": [P, P, P, I, I, I, I, I, P],
         "ra_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, P],
+        "ra_gemm_skinny_gated_bf16": [P, P, P, I, I, I, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P],
@@ -88,6 +89,7 @@ class HipOps:
         torch.backends.cudnn.allow_tf32 = False
         self.decode_split_tokens = 0         # keys per split of the decode attention; 0: by batch size
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
+        self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -274,6 +276,22 @@ class HipOps:
         self._check(self.lib.ra_gemm_nt(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(x.dtype),
                                         _code(out_dtype), self._stream()), "gemm_nt")
         return y
+
+    def linear_silu_mul(self, x, w_gate_up):
+        """silu(x @ Wg^T) * (x @ Wu^T) for w_gate_up = [Wg; Wu]: one kernel for few rows, else two."""
+        self._want(x, "x", dims=2)
+        self._want(w_gate_up, "gate-up weight", x.dtype, 2)
+        M, K = x.shape
+        I = w_gate_up.shape[0] // 2
+        if w_gate_up.shape[1] != K or w_gate_up.shape[0] != 2 * I:
+            raise KernelError(f"linear_silu_mul: x {tuple(x.shape)}, weight {tuple(w_gate_up.shape)}")
+        out = torch.empty(M, I, dtype=x.dtype, device=self.device)
+        if x.dtype == torch.bfloat16 and 0 < M <= self.gated_skinny_rows and K % 8 == 0:
+            self._check(self.lib.ra_gemm_skinny_gated_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K,
+                                                           self._stream()), "gemm_skinny_gated")
+            return out
+        self.silu_mul(self.linear(x, w_gate_up), out)
+        return out
 
     # ------------------------------------------------------------------ attention
     def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):

@@ -29,9 +29,7 @@ class SwiGLU:
 
     def forward(self, x, step=None):
         ops = self.rt.ops
-        gu = ops.linear(x, self.w_gate_up)                 # [T, 2I], gate first
-        a = self.rt.empty(x.shape[0], self.inter)
-        ops.silu_mul(gu, a)
+        a = ops.linear_silu_mul(x, self.w_gate_up)         # [T, I] = silu(gate) * up, gate rows first
         return ops.linear(a, self.w_down)
 
 

@@ -172,6 +172,26 @@ def test_linear(ops, dtype, out_dtype, M, N, K):
         torch.testing.assert_close(y.double(), want, atol=3e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 160, 96), (3, 200, 120), (8, 1000, 256), (20, 48, 64), (8, 24, 40)])
+def test_linear_silu_mul(ops, ref, dtype, M, I, K):
+    x = rnd(M, K, dtype=dtype, seed=43)
+    w = rnd(2 * I, K, dtype=dtype, seed=44, scale=0.2)
+    a, b = ops.linear_silu_mul(x, w), ref.linear_silu_mul(x, w)
+    assert a.shape == (M, I)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,K", [(331, 120), (48, 1000), (1000, 264)])
+def test_skinny_product_fp32_out(ops, M, N, K):
+    """bf16 rows times bf16 weights with fp32 results (the output head's product)."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=45)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=46, scale=0.1)
+    y = ops.linear(x, w, out_dtype=torch.float32)
+    torch.testing.assert_close(y.double(), x.double() @ w.double().t(), atol=1e-4 * K ** 0.5, rtol=1e-5)
+
+
 def test_linear_fp32_is_true_fp32(ops):
     """Inputs 1 + 2^-12 round to 1 in bf16 and tf32; a true 32-bit product keeps the 2^-11 per term."""
     K = 64

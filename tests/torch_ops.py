@@ -99,6 +99,13 @@ class TorchOps:
     def linear(self, x, w, out_dtype=None):
         return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
 
+    # rollout/monkey_patch/qwen3.py:20-22
+    def linear_silu_mul(self, x, w_gate_up):
+        gu = self.linear(x, w_gate_up)
+        out = torch.empty(x.shape[0], w_gate_up.shape[0] // 2, dtype=x.dtype, device=x.device)
+        self.silu_mul(gu, out)
+        return out
+
     # rollout/attention.py:126-139 over the tables of rollout/cache.py:282-328,
     # gathered as opd/test_parallel.py:14-42 does
     def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
