@@ -11,34 +11,42 @@
 // BUILD-VARIANTS: PRE_PART=0 PRE_PART=1 PRE_PART=2 PRE_PART=3 PRE_API=1
 //
 // One workgroup of four waves per (q tile of 64 rows, query head); wave w owns rows 16w..16w+15.
-// Per pass a tile of BN keys is staged in LDS: K row-major (padded rows), V transposed.
+// Per pass a tile of BN keys sits in LDS, K and V both row-major with padded rows; the next
+// tile's rows are already on their way from the cache into registers while this one is used.
 //  scores  S^T = K Q^T by MFMA 16x16x32 bf16: A = K tile rows from LDS, B = the wave's 16
 //          query rows held in registers. Lane (n, g) gets query n, keys 4g..4g+3 of each
 //          16-key tile.
 //  P.V     O^T += V^T P^T by the same MFMA. The contraction runs over keys in the order the
 //          lanes already hold them: k-slot (g, e) of a 32-key block is key 16*(e/4) + 4g + e%4,
-//          so P goes from the softmax registers straight into the B operand, and the A
-//          operand is two 8-byte reads of the transposed V tile.
+//          so P goes from the softmax registers straight into the B operand. The A operand,
+//          V^T, comes from the row-major V tile through the transposing LDS read of gfx950
+//          (ds_read_b64_tr_b16): within 16 lanes, lane l receives element l%4 of the 8 bytes
+//          addressed by lanes l/4, l/4+4, l/4+8, l/4+12. Lane l' therefore points at key
+//          4g + l'/4 (and 16 more for the second half), columns 16dt + 4(l'%4)..+3, and lane n
+//          ends up with column 16dt + n of keys 4g..4g+3.
 // A trailing 16 of D is a 16x16x32 step with the upper k half zero (one MFMA shape per chain).
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 #define PRE_BM 64
 
 #ifdef PRE_PART
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+// two floats to two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
-    return (uint32_t)f2bf_bits(a) | ((uint32_t)f2bf_bits(b) << 16);
+    const float2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
-union PK8 {
-    bf16x8_t v;
-    uint32_t w[4];
-    uint2 h[2];
-};
+typedef short short8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+typedef short4_t __attribute__((address_space(3))) * lds_short4_ptr;
 
 template <int D16>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
@@ -47,20 +55,37 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ tiles,       // [n_tiles][2]: request number, first row of the tile within it
-    int Hq, int Hkv, int P, float scale, int window) {
+    int n_tiles, int Hq, int Hkv, int P, float scale, int window) {
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;
     constexpr bool TAIL16 = (D % 32) != 0;
     constexpr int BN = (D <= 128) ? 64 : 32;            // keys per pass
-    constexpr int KS = D + 8;                           // K tile row stride (elements): 16 bytes of padding
-    constexpr int VS = BN + 2;                          // V^T tile row stride (elements)
+    constexpr int KS = D + 8;                           // K tile row stride (elements): rows shift by 4 banks
+    constexpr int VS = D + 16;                          // V tile row stride: rows shift by 8 banks (transposing reads)
     constexpr int LPR = D / 8;                          // threads that load one row (16 bytes each)
+    constexpr int NLD = (BN * LPR + 255) / 256;         // 16-byte pieces of K (and of V) per thread per tile
 
     __shared__ __attribute__((aligned(16))) uint16_t k_s[BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t vt_s[D * VS];
-    __shared__ int row_s[BN];
+    __shared__ __attribute__((aligned(16))) uint16_t v_s[BN * VS];
 
-    const int tile = blockIdx.x, head = blockIdx.y;
+    // Workgroups go to the 8 XCDs round-robin by their number, and each XCD has an L2 of its own:
+    // all workgroups of one kv head are sent to the same XCD, so that its keys and values are
+    // fetched into one L2 only (when the kv heads divide evenly among the XCDs).
+    int tile, head;
+    {
+        const int wg = blockIdx.x, per_head = n_tiles;
+        if (Hkv % 8 == 0) {
+            const int xcd = wg & 7, slot = wg >> 3;              // slot-th workgroup of this XCD
+            const int G_ = Hq / Hkv;
+            const int hh = slot / per_head;                      // which of this XCD's query heads
+            const int kv_local = hh / G_;                        // kv heads xcd, xcd+8, ... belong here
+            head = (kv_local * 8 + xcd) * G_ + hh % G_;
+            tile = slot % per_head;
+        } else {
+            head = wg / per_head;
+            tile = wg % per_head;
+        }
+    }
     const int seg = tiles[2 * tile], q_off = tiles[2 * tile + 1];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int kvh = head / (Hq / Hkv);
@@ -94,33 +119,60 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     int first_key = start;
     if (window > 0 && tile_first_pos - window + 1 > first_key) first_key = tile_first_pos - window + 1;
 
+    const float scale2 = scale * 1.44269504088896340736f;
+    // positions of the first and last row of this wave (wave-uniform, for skipping the mask)
+    const int wave_first_pos = pos0 + q_off + wave * 16;
+    const int wave_last_pos = wave_first_pos + 15;
     float m_run = -INFINITY, l_run = 0.f;
     float4_t acc[D16];
 #pragma unroll
     for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int c0 = (first_key / BN) * BN; c0 <= tile_last_pos; c0 += BN) {
-        // ---- stage the key tile: rows, then K row-major and V transposed
-        if (tid < BN) {
-            const int kpos = min(max(c0 + tid, first_key), tile_last_pos);
-            const int idx = kpos - start;
-            row_s[tid] = pt[idx / P] * P + idx % P;
-        }
-        __syncthreads();
-        for (int e = tid; e < BN * LPR; e += 256) {
-            const int key = e / LPR, c8 = (e % LPR) * 8;
-            const size_t src = ((size_t)row_s[key] * Hkv + kvh) * D + c8;
-            const uint4 kk = *reinterpret_cast<const uint4*>(k_pool + src);
-            *reinterpret_cast<uint4*>(&k_s[key * KS + c8]) = kk;
-            const uint4 vv = *reinterpret_cast<const uint4*>(v_pool + src);
-            const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+    // what each thread moves per tile: NLD 16-byte pieces of K and of V
+    uint4_t kreg[NLD], vreg[NLD];                        // native vectors: they stay in registers
+    int ld_key[NLD], ld_c8[NLD];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                vt_s[(c8 + 2 * i) * VS + key] = (uint16_t)(w[i] & 0xffffu);
-                vt_s[(c8 + 2 * i + 1) * VS + key] = (uint16_t)(w[i] >> 16);
+    for (int i = 0; i < NLD; ++i) {
+        const int e = min(tid + i * 256, BN * LPR - 1);    // surplus threads repeat the last piece
+        ld_key[i] = e / LPR;
+        ld_c8[i] = (e % LPR) * 8;
+    }
+    // cache row of key position kp (clamped into what this tile may read, so every address is valid)
+    const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
+#define ROW_OF(kp)                                                                  \
+    ([&]() {                                                                        \
+        const int idx_ = min(max((kp), first_key), tile_last_pos) - start;          \
+        const int pi_ = p_shift >= 0 ? (idx_ >> p_shift) : (idx_ / P);              \
+        return pt[pi_] * P + (idx_ - pi_ * P);                                      \
+    }())
+    const int c_first = (first_key / BN) * BN;
+    int row_next[NLD];                                   // rows of the tile that is fetched next
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int r0 = ROW_OF(c_first + ld_key[i]);
+        const size_t src = ((size_t)r0 * Hkv + kvh) * D + ld_c8[i];
+        kreg[i] = *reinterpret_cast<const uint4_t*>(k_pool + src);
+        vreg[i] = *reinterpret_cast<const uint4_t*>(v_pool + src);
+        row_next[i] = ROW_OF(c_first + BN + ld_key[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        *reinterpret_cast<uint4_t*>(&k_s[ld_key[i] * KS + ld_c8[i]]) = kreg[i];
+        *reinterpret_cast<uint4_t*>(&v_s[ld_key[i] * VS + ld_c8[i]]) = vreg[i];
+    }
+    __syncthreads();
+
+    for (int c0 = c_first; c0 <= tile_last_pos; c0 += BN) {
+        const bool has_next = c0 + BN <= tile_last_pos;
+        if (has_next) {                                  // the next tile travels while this one is used,
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {              // and the page lookups of the one after it
+                const size_t src = ((size_t)row_next[i] * Hkv + kvh) * D + ld_c8[i];
+                kreg[i] = *reinterpret_cast<const uint4_t*>(k_pool + src);
+                vreg[i] = *reinterpret_cast<const uint4_t*>(v_pool + src);
+                row_next[i] = ROW_OF(c0 + 2 * BN + ld_key[i]);
             }
         }
-        __syncthreads();
 
         // ---- scores of the wave's 16 rows against the BN keys
         float4_t cs[BN / 16];
@@ -141,17 +193,32 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             cs[st] = c;
         }
         MFMA_SETTLE();
+        // Scores in the base-2 domain: s2 = (q.k) * scale * log2(e), so that p = 2^(s2 - m).
         float s[BN / 16][4];
         float mx = -INFINITY;
+        // a tile that lies wholly below every row of the wave and inside every window needs no mask
+        const bool need_mask = (c0 + BN - 1 > wave_first_pos) || (c0 < first_key) ||
+                               (window > 0 && c0 <= wave_last_pos - window);
+        if (need_mask) {
 #pragma unroll
-        for (int st = 0; st < BN / 16; ++st) {
+            for (int st = 0; st < BN / 16; ++st) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int kpos = c0 + st * 16 + 4 * g + i;
-                bool ok = kpos >= first_key && kpos <= pos_q;
-                if (window > 0) ok = ok && kpos > pos_q - window;
-                s[st][i] = ok ? cs[st][i] * scale : -INFINITY;
-                mx = fmaxf(mx, s[st][i]);
+                for (int i = 0; i < 4; ++i) {
+                    const int kpos = c0 + st * 16 + 4 * g + i;
+                    bool ok = kpos >= first_key && kpos <= pos_q;
+                    if (window > 0) ok = ok && kpos > pos_q - window;
+                    s[st][i] = ok ? cs[st][i] * scale2 : -INFINITY;
+                    mx = fmaxf(mx, s[st][i]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int st = 0; st < BN / 16; ++st) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s[st][i] = cs[st][i] * scale2;
+                    mx = fmaxf(mx, s[st][i]);
+                }
             }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -164,44 +231,52 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         for (int st = 0; st < BN / 16; ++st)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                s[st][i] = (s[st][i] == -INFINITY) ? 0.f : __expf(s[st][i] - m_use);
+                s[st][i] = __builtin_amdgcn_exp2f(s[st][i] - m_use);      // 2^(-inf) = 0 for masked keys
                 lsum += s[st][i];
             }
         lsum += __shfl_xor(lsum, 16, 64);
         lsum += __shfl_xor(lsum, 32, 64);
-        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_use);
+        const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_use);
         l_run = l_run * alpha + lsum;
-        m_run = m_new;
-#pragma unroll
-        for (int dt = 0; dt < D16; ++dt) {
-            acc[dt][0] *= alpha;
-            acc[dt][1] *= alpha;
-            acc[dt][2] *= alpha;
-            acc[dt][3] *= alpha;
-        }
-
-        // ---- O^T += V^T P^T, 32 keys per MFMA
-#pragma unroll
-        for (int b = 0; b < BN / 32; ++b) {
-            PK8 pb;
-            pb.w[0] = pack2(s[2 * b][0], s[2 * b][1]);
-            pb.w[1] = pack2(s[2 * b][2], s[2 * b][3]);
-            pb.w[2] = pack2(s[2 * b + 1][0], s[2 * b + 1][1]);
-            pb.w[3] = pack2(s[2 * b + 1][2], s[2 * b + 1][3]);
+        if (__any(m_new != m_run)) {                     // some row's maximum moved: rescale what is summed so far
 #pragma unroll
             for (int dt = 0; dt < D16; ++dt) {
-                const uint16_t* vr = &vt_s[(dt * 16 + n) * VS + 32 * b + 4 * g];
-                PK8 va;
-                va.w[0] = *reinterpret_cast<const uint32_t*>(vr);
-                va.w[1] = *reinterpret_cast<const uint32_t*>(vr + 2);
-                va.w[2] = *reinterpret_cast<const uint32_t*>(vr + 16);
-                va.w[3] = *reinterpret_cast<const uint32_t*>(vr + 18);
-                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, acc[dt], 0, 0, 0);
+                acc[dt][0] *= alpha;
+                acc[dt][1] *= alpha;
+                acc[dt][2] *= alpha;
+                acc[dt][3] *= alpha;
+            }
+        }
+        m_run = m_new;
+
+        // ---- O^T += V^T P^T, 32 keys per MFMA; V^T through the transposing LDS read
+#pragma unroll
+        for (int b = 0; b < BN / 32; ++b) {
+            const uint4_t pw = {pack2(s[2 * b][0], s[2 * b][1]), pack2(s[2 * b][2], s[2 * b][3]),
+                                pack2(s[2 * b + 1][0], s[2 * b + 1][1]), pack2(s[2 * b + 1][2], s[2 * b + 1][3])};
+            const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, pw);
+            // this lane's address as lane l' = n of its group: key 32b + 4g + n/4, columns 4(n%4)..+3
+            const uint16_t* vr = &v_s[(32 * b + 4 * g + (n >> 2)) * VS + 4 * (n & 3)];
+#pragma unroll
+            for (int dt = 0; dt < D16; ++dt) {
+                const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + dt * 16));
+                const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + 16 * VS + dt * 16));
+                const short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), pb, acc[dt], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                 // every wave is done with this tile
+        if (has_next) {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                *reinterpret_cast<uint4_t*>(&k_s[ld_key[i] * KS + ld_c8[i]]) = kreg[i];
+                *reinterpret_cast<uint4_t*>(&v_s[ld_key[i] * VS + ld_c8[i]]) = vreg[i];
             }
         }
         __syncthreads();
     }
 
+#undef ROW_OF
     MFMA_SETTLE();
     // ---- acc[dt][i] = O^T[d = 16dt + 4g + i][query n]
     if (q_ok) {
@@ -223,12 +298,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, dim3 grid, hipStream_t st, const bf16* q, bf16* out,
                                               const bf16* kp, const bf16* vp, const int* pt,
                                               const int* cup, const int* kvs, const int* cuq,
-                                              const int* qs, const int* tiles, int Hq, int Hkv, int P,
-                                              float scale, int window) {
+                                              const int* qs, const int* tiles, int n_tiles, int Hq,
+                                              int Hkv, int P, float scale, int window) {
 #define PRE_CASE(N)                                                                               \
     case N:                                                                                       \
         hipLaunchKernelGGL(attn_prefill_kernel<N>, grid, dim3(256), 0, st, q, out, kp, vp, pt, cup, \
-                           kvs, cuq, qs, tiles, Hq, Hkv, P, scale, window);                       \
+                           kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window);              \
         return RA_OK;
     switch (D16) {
         PRE_CASE(4 * PRE_PART + 1) PRE_CASE(4 * PRE_PART + 2) PRE_CASE(4 * PRE_PART + 3)
@@ -242,7 +317,7 @@ extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, dim3 grid, hipStream_t s
 #ifdef PRE_API
 #define PRE_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
     const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs,    \
-    const int* tiles, int Hq, int Hkv, int P, float scale, int window
+    const int* tiles, int n_tiles, int Hq, int Hkv, int P, float scale, int window
 extern "C" int ra_pre_part_0(PRE_PART_ARGS);
 extern "C" int ra_pre_part_1(PRE_PART_ARGS);
 extern "C" int ra_pre_part_2(PRE_PART_ARGS);
@@ -256,16 +331,17 @@ extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k
                                          const int* q_start, const int* tiles, int n_tiles, int Hq,
                                          int Hkv, int D, int P, float scale, int window, void* stream) {
     if (n_tiles <= 0) return RA_OK;
-    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || Hq > 65535 || P <= 0)
+    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 ||
+        (long long)n_tiles * Hq > 0x7fffffffLL)
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid(n_tiles, Hq);
+    dim3 grid(n_tiles * Hq);
     const int d16 = D / 16;
     int rc;
 #define GO(k)                                                                                      \
     rc = ra_pre_part_##k(d16, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tiles, \
-                         Hq, Hkv, P, scale, window)
+                         n_tiles, Hq, Hkv, P, scale, window)
     switch ((d16 - 1) / 4) {
         case 0: GO(0); break;
         case 1: GO(1); break;

@@ -69,9 +69,13 @@ class StepBatch:
 PREFILL_TILE_ROWS = 64      # query rows per workgroup of the prefill attention kernel
 
 
-def prefill_tiles(q_lens):
-    """(request number, first row) of every tile of PREFILL_TILE_ROWS rows, for requests with more than one token."""
-    return [(i, off) for i, q in enumerate(q_lens) if q != 1 for off in range(0, q, PREFILL_TILE_ROWS)]
+def prefill_tiles(q_lens, q_starts=None):
+    """(request number, first row) of every tile of PREFILL_TILE_ROWS rows, for requests with more
+    than one token; tiles that read the most keys come first, so the longest work starts earliest."""
+    tiles = [(i, off) for i, q in enumerate(q_lens) if q != 1 for off in range(0, q, PREFILL_TILE_ROWS)]
+    if q_starts is not None:
+        tiles.sort(key=lambda t: -(int(q_starts[t[0]]) + t[1]))
+    return tiles
 
 
 class StepBuilder:
@@ -156,7 +160,7 @@ class StepBuilder:
             self._put(f"cu_pages{g}", gt.cu_pages)
             self._put(f"kv_start{g}", gt.kv_start)
             self._put(f"page_table{g}", gt.page_table)
-        tiles = prefill_tiles(tables.q_lens)
+        tiles = prefill_tiles(tables.q_lens, tables.q_start)
         if tiles:
             self._put("prefill_tiles", np.asarray(tiles, dtype=np.int32).reshape(-1))
         # one copy for the small tables, one per group for the used part of its page table

@@ -225,7 +225,7 @@ def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
                  prefill_toks=i32([t for i in pre for t in range(cu_q[i], cu_q[i + 1])]) if both else None,
                  prefill_segs=pre)
     from return_amd.engine.batch import prefill_tiles
-    tiles = prefill_tiles(q_lens)
+    tiles = prefill_tiles(q_lens, q_starts)
     extra.update(n_prefill_tiles=len(tiles), prefill_tiles=i32(tiles) if tiles else None)
     return types.SimpleNamespace(**extra, n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
                                  seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
