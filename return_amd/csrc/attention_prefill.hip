@@ -62,11 +62,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     constexpr int BN = (D <= 128) ? 64 : 32;            // keys per pass
     constexpr int KS = D + 8;                           // K tile row stride (elements): rows shift by 4 banks
     constexpr int VS = D + 16;                          // V tile row stride: rows shift by 8 banks (transposing reads)
-    constexpr int LPR = D / 8;                          // threads that load one row (16 bytes each)
-    constexpr int NLD = (BN * LPR + 255) / 256;         // 16-byte pieces of K (and of V) per thread per tile
+    constexpr int LPR = D / 8;                          // 16-byte pieces in one row
+    constexpr int TPK = 256 / BN;                       // threads that share the loading of one key row
+    constexpr int NLD = (LPR + TPK - 1) / TPK;          // pieces of K (and of V) per thread per tile
 
-    __shared__ __attribute__((aligned(16))) uint16_t k_s[BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t v_s[BN * VS];
+    // two tiles: one is used while the next is written
+    __shared__ __attribute__((aligned(16))) uint16_t k_s[2][BN * KS];
+    __shared__ __attribute__((aligned(16))) uint16_t v_s[2][BN * VS];
 
     // Workgroups go to the 8 XCDs round-robin by their number, and each XCD has an L2 of its own:
     // all workgroups of one kv head are sent to the same XCD, so that its keys and values are
@@ -77,13 +79,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         if (Hkv % 8 == 0) {
             const int xcd = wg & 7, slot = wg >> 3;              // slot-th workgroup of this XCD
             const int G_ = Hq / Hkv;
-            const int hh = slot / per_head;                      // which of this XCD's query heads
+            const int heads_here = Hq >> 3;
+            const int hh = slot % heads_here;                    // which of this XCD's query heads
             const int kv_local = hh / G_;                        // kv heads xcd, xcd+8, ... belong here
             head = (kv_local * 8 + xcd) * G_ + hh % G_;
-            tile = slot % per_head;
+            tile = slot / heads_here;                            // tiles come longest first: all heads' long ones start early
         } else {
-            head = wg / per_head;
-            tile = wg % per_head;
+            head = wg % Hq;
+            tile = wg / Hq;
         }
     }
     const int seg = tiles[2 * tile], q_off = tiles[2 * tile + 1];
@@ -128,15 +131,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
     for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // what each thread moves per tile: NLD 16-byte pieces of K and of V
+    // what each thread moves per tile: its key row's pieces my_sub, my_sub + TPK, ... of K and of V
     uint4_t kreg[NLD], vreg[NLD];                        // native vectors: they stay in registers
-    int ld_key[NLD], ld_c8[NLD];
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-        const int e = min(tid + i * 256, BN * LPR - 1);    // surplus threads repeat the last piece
-        ld_key[i] = e / LPR;
-        ld_c8[i] = (e % LPR) * 8;
-    }
+    const int my_key = tid / TPK, my_sub = tid % TPK;
     // cache row of key position kp (clamped into what this tile may read, so every address is valid)
     const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
 #define ROW_OF(kp)                                                                  \
@@ -145,32 +142,49 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         const int pi_ = p_shift >= 0 ? (idx_ >> p_shift) : (idx_ / P);              \
         return pt[pi_] * P + (idx_ - pi_ * P);                                      \
     }())
-    const int c_first = (first_key / BN) * BN;
-    int row_next[NLD];                                   // rows of the tile that is fetched next
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-        const int r0 = ROW_OF(c_first + ld_key[i]);
-        const size_t src = ((size_t)r0 * Hkv + kvh) * D + ld_c8[i];
-        kreg[i] = *reinterpret_cast<const uint4_t*>(k_pool + src);
-        vreg[i] = *reinterpret_cast<const uint4_t*>(v_pool + src);
-        row_next[i] = ROW_OF(c_first + BN + ld_key[i]);
+#define FETCH_ROW(row_)                                                             \
+    {                                                                               \
+        const size_t base_ = ((size_t)(row_) * Hkv + kvh) * D;                      \
+        _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                           \
+            const int p_ = my_sub + TPK * i;                                        \
+            if (p_ < LPR) {                                                         \
+                kreg[i] = *reinterpret_cast<const uint4_t*>(k_pool + base_ + 8 * p_); \
+                vreg[i] = *reinterpret_cast<const uint4_t*>(v_pool + base_ + 8 * p_); \
+            }                                                                       \
+        }                                                                           \
     }
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-        *reinterpret_cast<uint4_t*>(&k_s[ld_key[i] * KS + ld_c8[i]]) = kreg[i];
-        *reinterpret_cast<uint4_t*>(&v_s[ld_key[i] * VS + ld_c8[i]]) = vreg[i];
+#define STAGE_TO(buf_)                                                              \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                               \
+        const int p_ = my_sub + TPK * i;                                            \
+        if (p_ < LPR) {                                                             \
+            *reinterpret_cast<uint4_t*>(&k_s[buf_][my_key * KS + 8 * p_]) = kreg[i]; \
+            *reinterpret_cast<uint4_t*>(&v_s[buf_][my_key * VS + 8 * p_]) = vreg[i]; \
+        }                                                                           \
+    }
+    const int c_first = (first_key / BN) * BN;
+    int row_next;                                        // row of this thread's key in the tile fetched next
+    {
+        const int r0 = ROW_OF(c_first + my_key);
+        row_next = ROW_OF(c_first + BN + my_key);
+        FETCH_ROW(r0)
+        STAGE_TO(0)
+        FETCH_ROW(row_next)                              // tile 1 (or a repeat of valid rows if there is none)
+        row_next = ROW_OF(c_first + 2 * BN + my_key);
     }
     __syncthreads();
 
-    for (int c0 = c_first; c0 <= tile_last_pos; c0 += BN) {
-        const bool has_next = c0 + BN <= tile_last_pos;
-        if (has_next) {                                  // the next tile travels while this one is used,
-#pragma unroll
-            for (int i = 0; i < NLD; ++i) {              // and the page lookups of the one after it
-                const size_t src = ((size_t)row_next[i] * Hkv + kvh) * D + ld_c8[i];
-                kreg[i] = *reinterpret_cast<const uint4_t*>(k_pool + src);
-                vreg[i] = *reinterpret_cast<const uint4_t*>(v_pool + src);
-                row_next[i] = ROW_OF(c0 + 2 * BN + ld_key[i]);
+    int it = 0;
+    for (int c0 = c_first; c0 <= tile_last_pos; c0 += BN, ++it) {
+        const int cur = it & 1;
+        const uint16_t* k_cur = k_s[cur];
+        const uint16_t* v_cur = v_s[cur];
+        if (c0 + BN <= tile_last_pos) {
+            // the next tile, asked for one pass ago, goes into the other buffer (which every wave left
+            // at the last barrier); then the tile after it is asked for
+            STAGE_TO(cur ^ 1)
+            if (c0 + 2 * BN <= tile_last_pos) {
+                FETCH_ROW(row_next)
+                row_next = ROW_OF(c0 + 3 * BN + my_key);
             }
         }
 
@@ -179,7 +193,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
         for (int st = 0; st < BN / 16; ++st) {
             float4_t c = {0.f, 0.f, 0.f, 0.f};
-            const uint16_t* kr = &k_s[(st * 16 + n) * KS];
+            const uint16_t* kr = &k_cur[(st * 16 + n) * KS];
 #pragma unroll
             for (int j = 0; j < D32; ++j) {
                 const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(kr + 32 * j + 8 * g);
@@ -256,7 +270,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                                 pack2(s[2 * b + 1][0], s[2 * b + 1][1]), pack2(s[2 * b + 1][2], s[2 * b + 1][3])};
             const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, pw);
             // this lane's address as lane l' = n of its group: key 32b + 4g + n/4, columns 4(n%4)..+3
-            const uint16_t* vr = &v_s[(32 * b + 4 * g + (n >> 2)) * VS + 4 * (n & 3)];
+            const uint16_t* vr = &v_cur[(32 * b + 4 * g + (n >> 2)) * VS + 4 * (n & 3)];
 #pragma unroll
             for (int dt = 0; dt < D16; ++dt) {
                 const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + dt * 16));
@@ -265,17 +279,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), pb, acc[dt], 0, 0, 0);
             }
         }
-        __syncthreads();                                 // every wave is done with this tile
-        if (has_next) {
-#pragma unroll
-            for (int i = 0; i < NLD; ++i) {
-                *reinterpret_cast<uint4_t*>(&k_s[ld_key[i] * KS + ld_c8[i]]) = kreg[i];
-                *reinterpret_cast<uint4_t*>(&v_s[ld_key[i] * VS + ld_c8[i]]) = vreg[i];
-            }
-        }
-        __syncthreads();
+        __syncthreads();                                 // every wave is done with this tile; the next one is complete
     }
 
+#undef FETCH_ROW
+#undef STAGE_TO
 #undef ROW_OF
     MFMA_SETTLE();
     // ---- acc[dt][i] = O^T[d = 16dt + 4g + i][query n]
