@@ -61,6 +61,7 @@ def _declare(lib):
         "ra_gemm_nt": [P, P, P, I, I, I, I, I, P],
         "ra_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, P],
         "ra_gemm_skinny_gated_bf16": [P, P, P, I, I, I, P],
+        "ra_gemm_mfma_bf16": [P, P, P, I, I, I, I, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P],
@@ -90,6 +91,7 @@ class HipOps:
         self.decode_split_tokens = 0         # keys per split of the decode attention; 0: by batch size
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
+        self.own_gemm = False                # True: bf16 products of many rows use the hand-written MFMA kernel
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -97,7 +99,7 @@ class HipOps:
         if K % 8 or M > 64:
             return False
         if out_dtype == torch.float32:
-            return True                      # the library has no bf16-in, fp32-out product
+            return M <= 16                   # more rows: the tiled MFMA product (the library has no bf16-in, fp32-out product)
         return M <= 4 or (M <= 16 and N * K <= (32 << 20))
 
     # ------------------------------------------------------------------ helpers
@@ -270,8 +272,13 @@ class HipOps:
             self._check(self.lib.ra_gemm_skinny_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
                                                      self.skinny_max_grid, self._stream()), "gemm_skinny")
             return y
-        if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and M > 0:
+        if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and M > 0 and not self.own_gemm:
             return torch.matmul(x, w.t())          # library product, as the reference's F.linear
+        if x.dtype == torch.bfloat16 and M > 0 and K % 8 == 0:
+            y = torch.empty(M, N, dtype=out_dtype, device=self.device)
+            self._check(self.lib.ra_gemm_mfma_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
+                                                   self._stream()), "gemm_mfma")
+            return y
         y = torch.empty(M, N, dtype=out_dtype, device=self.device)
         self._check(self.lib.ra_gemm_nt(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(x.dtype),
                                         _code(out_dtype), self._stream()), "gemm_nt")

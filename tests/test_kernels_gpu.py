@@ -192,6 +192,25 @@ def test_skinny_product_fp32_out(ops, M, N, K):
     torch.testing.assert_close(y.double(), x.double() @ w.double().t(), atol=1e-4 * K ** 0.5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(65, 331, 120), (128, 128, 32), (129, 257, 264), (300, 1000, 512), (70, 48, 8)])
+def test_tiled_mfma_product(ops, out_dtype, M, N, K):
+    """The hand-written tiled product for many rows, edges in every dimension."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=47)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=48, scale=0.1)
+    ops.own_gemm = True
+    try:
+        y = ops.linear(x, w, out_dtype=out_dtype)
+    finally:
+        ops.own_gemm = False
+    want = x.double() @ w.double().t()
+    assert y.dtype == out_dtype
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(y.double(), want, atol=1e-4 * K ** 0.5, rtol=1e-5)
+    else:
+        torch.testing.assert_close(y.double(), want, atol=3e-2, rtol=2e-2)
+
+
 def test_linear_fp32_is_true_fp32(ops):
     """Inputs 1 + 2^-12 round to 1 in bf16 and tf32; a true 32-bit product keeps the 2^-11 per term."""
     K = 64
