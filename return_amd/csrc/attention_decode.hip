@@ -12,24 +12,32 @@
 // One wave per (request, kv head, split), 64 keys per pass.
 //  scores  S^T = K Q^T by MFMA 16x16x32 bf16, the key tile as A operand read straight from
 //          the cache: lane (n, g) loads the 16 bytes d = 32j + 8g .. +7 of key n, so the four
-//          lane groups of a key read 64 contiguous bytes per load. A trailing 16 of D is one
-//          more step of the same MFMA with the upper half of k zero (an accumulation chain
-//          that mixed 16x16x32 and 16x16x16 lost the last 16x16x32 term on gfx950, so one
-//          shape is used throughout). Lane (n, g) ends up with query head n, keys 4g..4g+3
-//          of each tile.
-//  P.V     on the vector unit: D/8 lanes share a key's value row (16 bytes each), so one load
-//          instruction fetches 64/(D/8) keys; every lane accumulates its 8 columns over the
-//          keys it sees, and the lanes' partial sums are added through LDS at the end.
+//          lane groups of a key read 64 contiguous bytes per load; the B operand holds the
+//          group's query heads (up to 16) the same way. A trailing 16 of D is one more step of
+//          the same MFMA with the upper half of k zero (an accumulation chain that mixed
+//          16x16x32 and 16x16x16 lost the last 16x16x32 term on gfx950, so one shape is used
+//          throughout). Lane (n, g) ends up with query head n, keys 4g..4g+3 of each tile.
+//  P.V     O^T += V^T P^T by the same MFMA: the value rows go through LDS (16-byte pieces in,
+//          transposing reads ds_read_b64_tr_b16 out: within 16 lanes, lane l receives element
+//          l%4 of the 8 bytes addressed by lanes l/4, l/4+4, l/4+8, l/4+12), and P goes from
+//          the softmax registers straight into the B operand because the contraction runs over
+//          keys in the order the lanes already hold them (k-slot (g, e) of a 32-key block is
+//          key 16*(e/4) + 4g + e%4). The cost does not depend on how many heads share a kv head.
 // BUILD-VARIANTS: DEC_PART=0 DEC_PART=1 DEC_PART=2 DEC_PART=3 DEC_API=1
 // (each DEC_PART instantiates four head sizes; DEC_API holds the entry point and the merge)
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef short short8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef short4_t __attribute__((address_space(3))) * lds_short4_ptr;
 
 #define DEC_CHUNK 64          // keys per pass of a wave
-#define DEC_MAX_GROUP 16      // query heads per kv head (rows of the MFMA tile)
+#define DEC_MAX_GROUP 16      // query heads per kv head (columns of the MFMA tile)
 
 struct DecodeRange {
     int lo, hi;               // key positions of this split, inclusive; lo > hi: empty
@@ -50,13 +58,14 @@ __device__ __forceinline__ DecodeRange decode_range(int pos_q, int start, int wi
 }
 
 #ifdef DEC_PART
-union V16 {
-    uint4 u;
-    uint32_t w[4];
-};
+// two floats to two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const float2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
-template <int D16, int GMAX>
-__global__ __launch_bounds__(64) void attn_decode_kernel(
+template <int D16>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2 : 1))) void attn_decode_kernel(
     const bf16* __restrict__ q, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
     const int* __restrict__ page_table, const int* __restrict__ cu_pages,
@@ -65,15 +74,12 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     float scale, int window, int split_tokens, int max_splits) {
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;                 // full MFMA x32 steps
-    constexpr bool TAIL16 = (D % 32) != 0;      // one more step of 16
-    constexpr int LPR = D / 8;                  // lanes that share one value row
-    constexpr int KPI = 64 / LPR;               // keys per value load instruction
-    constexpr int NVI = (DEC_CHUNK + KPI - 1) / KPI;   // value load instructions per pass
+    constexpr bool TAIL16 = (D % 32) != 0;      // one more step, upper k half zero
+    constexpr int LPR = D / 8;                  // 16-byte pieces in one value row
+    constexpr int NVL = (DEC_CHUNK * LPR + 63) / 64;   // pieces of the value tile per lane
+    constexpr int VS = D + 16;                  // value tile row stride in LDS (elements): rows shift by 8 banks
 
-    __shared__ float p_s[DEC_CHUNK * DEC_MAX_GROUP];   // [key][query head]
-    __shared__ float alpha_s[DEC_MAX_GROUP];
-    __shared__ int row_s[DEC_CHUNK];
-    extern __shared__ float red_s[];                   // [KPI][G][D] at the end
+    __shared__ __attribute__((aligned(16))) uint16_t v_s[DEC_CHUNK * VS];
 
     const int di = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
     const int seg = seg_ids ? seg_ids[di] : di;
@@ -85,8 +91,9 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     const DecodeRange rg = decode_range(pos_q, start, window, split_tokens, sp);
     if (rg.lo > rg.hi) return;
     const int* pt = page_table + cu_pages[seg];
+    const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
 
-    // query operand: lane (n, g) holds head kvh*G+n, d = 32j + 8g .. +7 (and D-16+4g.. for the tail)
+    // query operand: lane (n, g) holds head kvh*G+n, d = 32j + 8g .. +7 (and D-16+8g.. for the tail)
     const bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8_t bq[D32 > 0 ? D32 : 1];
     bf16x8_t bq_tail = z8;
@@ -102,24 +109,19 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
         }
     }
 
-    // value stage: this lane's columns and its key slot within a load instruction
-    const int vkey = lane / LPR, vcol = (lane % LPR) * 8;
-    const bool v_active = lane < KPI * LPR;
-
+    const float scale2 = scale * 1.44269504088896340736f;      // scores in the base-2 domain
     float m_run = -INFINITY, l_run = 0.f;
-    float acc[GMAX][8];
+    float4_t acc[D16];                           // acc[dt][i] = O^T[d = 16dt + 4g + i][head n]
 #pragma unroll
-    for (int h = 0; h < GMAX; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
+    for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int c_begin = (rg.lo / DEC_CHUNK) * DEC_CHUNK;
     for (int c0 = c_begin; c0 <= rg.hi; c0 += DEC_CHUNK) {
         // row of this lane's key (clamped into the split so that every address is valid)
-        int kpos = min(max(c0 + lane, rg.lo), rg.hi);
+        const int kpos = min(max(c0 + lane, rg.lo), rg.hi);
         const int idx = kpos - start;
-        const int row = pt[idx / P] * P + idx % P;
-        row_s[lane] = row;
+        const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
+        const int row = pt[pi] * P + (idx - pi * P);
 
         // ---- K tiles straight into MFMA A operands
         bf16x8_t ak[4][D32 > 0 ? D32 : 1];
@@ -136,17 +138,19 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
                 if (g < 2) ak_tail[st] = *reinterpret_cast<const bf16x8_t*>(kp + (D - 16) + 8 * g);
             }
         }
-        __syncthreads();                           // row_s visible
-        // ---- V rows: issue all loads of the pass now
-        V16 vv[NVI];
+        // ---- V rows: 16-byte pieces, all loads of the pass issued now, then into LDS
+        uint4_t vv[NVL];
 #pragma unroll
-        for (int i = 0; i < NVI; ++i) {
-            const int k = i * KPI + vkey;
-            vv[i].u = make_uint4(0u, 0u, 0u, 0u);
-            if (v_active && k < DEC_CHUNK) {
-                const int r = row_s[k];
-                vv[i].u = *reinterpret_cast<const uint4*>(v_pool + ((size_t)r * Hkv + kvh) * D + vcol);
-            }
+        for (int i = 0; i < NVL; ++i) {
+            const int e = min(lane + 64 * i, DEC_CHUNK * LPR - 1);
+            const int r = __shfl(row, e / LPR, 64);
+            vv[i] = *reinterpret_cast<const uint4_t*>(v_pool + ((size_t)r * Hkv + kvh) * D + (e % LPR) * 8);
+        }
+        __syncthreads();                           // the previous pass has read its value tile
+#pragma unroll
+        for (int i = 0; i < NVL; ++i) {
+            const int e = min(lane + 64 * i, DEC_CHUNK * LPR - 1);
+            *reinterpret_cast<uint4_t*>(&v_s[(e / LPR) * VS + (e % LPR) * 8]) = vv[i];
         }
 
         // ---- scores
@@ -170,7 +174,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int kp_abs = c0 + st * 16 + 4 * g + i;
                 const bool ok = kp_abs >= rg.lo && kp_abs <= rg.hi;
-                s[st][i] = ok ? cs[st][i] * scale : -INFINITY;
+                s[st][i] = ok ? cs[st][i] * scale2 : -INFINITY;
                 mx = fmaxf(mx, s[st][i]);
             }
         }
@@ -182,111 +186,71 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
         for (int st = 0; st < 4; ++st)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = (s[st][i] == -INFINITY) ? 0.f : __expf(s[st][i] - m_new);
-                lsum += p;
-                p_s[(st * 16 + 4 * g + i) * DEC_MAX_GROUP + n] = p;
+                s[st][i] = __builtin_amdgcn_exp2f(s[st][i] - m_new);   // 2^(-inf) = 0 for masked keys
+                lsum += s[st][i];
             }
         lsum += __shfl_xor(lsum, 16, 64);
         lsum += __shfl_xor(lsum, 32, 64);
-        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
-        if (g == 0) alpha_s[n] = alpha;
+        const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
         l_run = l_run * alpha + lsum;
+        if (__any(m_new != m_run)) {
+#pragma unroll
+            for (int dt = 0; dt < D16; ++dt) {
+                acc[dt][0] *= alpha;
+                acc[dt][1] *= alpha;
+                acc[dt][2] *= alpha;
+                acc[dt][3] *= alpha;
+            }
+        }
         m_run = m_new;
-        __syncthreads();
+        __syncthreads();                           // the value tile is complete in LDS
 
-        // ---- P.V on the vector unit
+        // ---- O^T += V^T P^T, 32 keys per MFMA
 #pragma unroll
-        for (int h = 0; h < GMAX; ++h) {
-            const float a = alpha_s[h];
+        for (int b = 0; b < 2; ++b) {
+            const uint4_t pw = {pack2(s[2 * b][0], s[2 * b][1]), pack2(s[2 * b][2], s[2 * b][3]),
+                                pack2(s[2 * b + 1][0], s[2 * b + 1][1]), pack2(s[2 * b + 1][2], s[2 * b + 1][3])};
+            const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, pw);
+            // this lane's address as lane l' = n of its group: key 32b + 4g + n/4, columns 4(n%4)..+3
+            const uint16_t* vr = &v_s[(32 * b + 4 * g + (n >> 2)) * VS + 4 * (n & 3)];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[h][e] *= a;
-        }
-#pragma unroll
-        for (int i = 0; i < NVI; ++i) {
-            const int k = i * KPI + vkey;
-            if (v_active && k < DEC_CHUNK) {
-                float vf[8];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    vf[2 * e] = __uint_as_float(vv[i].w[e] << 16);
-                    vf[2 * e + 1] = __uint_as_float(vv[i].w[e] & 0xffff0000u);
-                }
-#pragma unroll
-                for (int h = 0; h < GMAX; ++h) {
-                    const float p = p_s[k * DEC_MAX_GROUP + h];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
-                }
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- add the key slots' partial sums through LDS, then write the split's result
-    if (v_active) {
-#pragma unroll
-        for (int h = 0; h < GMAX; ++h) {
-            if (h < G) {
-                float* r = red_s + ((size_t)vkey * G + h) * D + vcol;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) r[e] = acc[h][e];
+            for (int dt = 0; dt < D16; ++dt) {
+                const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + dt * 16));
+                const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + 16 * VS + dt * 16));
+                const short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), pb, acc[dt], 0, 0, 0);
             }
         }
     }
-    __syncthreads();
-    for (int e = lane; e < G * D; e += 64) {
-        float sum = 0.f;
+    MFMA_SETTLE();
+
+    // ---- partial results of this split: lane (n, g) holds head n, columns 16dt + 4g .. +3
+    if (n < G) {
+        float* pa = part_acc + (((size_t)di * Hq + (size_t)kvh * G + n) * max_splits + sp) * D;
 #pragma unroll
-        for (int ks = 0; ks < KPI; ++ks) sum += red_s[(size_t)ks * G * D + e];
-        const int h = e / D, d = e % D;
-        part_acc[(((size_t)di * Hq + (size_t)kvh * G + h) * max_splits + sp) * D + d] = sum;
-    }
-    if (g == 0 && n < G) {
-        float* pm = part_ml + (((size_t)di * Hq + (size_t)kvh * G + n) * max_splits + sp) * 2;
-        pm[0] = m_run;
-        pm[1] = l_run;
+        for (int dt = 0; dt < D16; ++dt) *reinterpret_cast<float4_t*>(pa + dt * 16 + 4 * g) = acc[dt];
+        if (g == 0) {
+            float* pm = part_ml + (((size_t)di * Hq + (size_t)kvh * G + n) * max_splits + sp) * 2;
+            pm[0] = m_run;
+            pm[1] = l_run;
+        }
     }
 }
-
-template <int D16, int GMAX>
-static void launch_decode(dim3 grid, size_t shmem, hipStream_t st, const bf16* q, float* pa,
-                          float* pm, const bf16* kp, const bf16* vp, const int* pt, const int* cup,
-                          const int* kvs, const int* cuq, const int* qs, const int* segs, int Hq,
-                          int Hkv, int P, float scale, int window, int split_tokens, int max_splits) {
-    hipLaunchKernelGGL((attn_decode_kernel<D16, GMAX>), grid, dim3(64), shmem, st, q, pa, pm, kp, vp,
-                       pt, cup, kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens,
-                       max_splits);
-}
-
-template <int D16>
-static int pick_group(int G, dim3 grid, size_t shmem, hipStream_t st, const bf16* q, float* pa,
-                      float* pm, const bf16* kp, const bf16* vp, const int* pt, const int* cup,
-                      const int* kvs, const int* cuq, const int* qs, const int* segs, int Hq, int Hkv,
-                      int P, float scale, int window, int split_tokens, int max_splits) {
-#define GO(GM)                                                                                     \
-    launch_decode<D16, GM>(grid, shmem, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs, segs, Hq, Hkv, \
-                           P, scale, window, split_tokens, max_splits)
-    if (G <= 4) GO(4);
-    else if (G <= 16) GO(16);
-    else return RA_ERR_ARG;
-#undef GO
-    return RA_OK;
-}
-
 
 #define DEC_CAT2(a, b) a##b
 #define DEC_CAT(a, b) DEC_CAT2(a, b)
 // head sizes 16*(4*DEC_PART+1) .. 16*(4*DEC_PART+4)
-extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, int G, dim3 grid, size_t shmem, hipStream_t st,
-                                              const bf16* q, float* pa, float* pm, const bf16* kp,
-                                              const bf16* vp, const int* pt, const int* cup,
-                                              const int* kvs, const int* cuq, const int* qs,
-                                              const int* segs, int Hq, int Hkv, int P, float scale,
-                                              int window, int split_tokens, int max_splits) {
-#define DEC_CASE(N)                                                                              \
-    case N:                                                                                      \
-        return pick_group<N>(G, grid, shmem, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs, segs, \
-                             Hq, Hkv, P, scale, window, split_tokens, max_splits);
+extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t st, const bf16* q, float* pa,
+                                              float* pm, const bf16* kp, const bf16* vp, const int* pt,
+                                              const int* cup, const int* kvs, const int* cuq,
+                                              const int* qs, const int* segs, int Hq, int Hkv, int P,
+                                              float scale, int window, int split_tokens,
+                                              int max_splits) {
+#define DEC_CASE(N)                                                                                \
+    case N:                                                                                        \
+        hipLaunchKernelGGL(attn_decode_kernel<N>, grid, dim3(64), 0, st, q, pa, pm, kp, vp, pt, cup, \
+                           kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits); \
+        return RA_OK;
     switch (D16) {
         DEC_CASE(4 * DEC_PART + 1) DEC_CASE(4 * DEC_PART + 2) DEC_CASE(4 * DEC_PART + 3)
         DEC_CASE(4 * DEC_PART + 4)
@@ -298,9 +262,9 @@ extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, int G, dim3 grid, size_t
 
 #ifdef DEC_API
 
-#define DEC_PART_ARGS int D16, int G, dim3 grid, size_t shmem, hipStream_t st, const bf16* q, float* pa, \
-    float* pm, const bf16* kp, const bf16* vp, const int* pt, const int* cup, const int* kvs,          \
-    const int* cuq, const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,   \
+#define DEC_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm,        \
+    const bf16* kp, const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq,   \
+    const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,                 \
     int split_tokens, int max_splits
 extern "C" int ra_dec_part_0(DEC_PART_ARGS);
 extern "C" int ra_dec_part_1(DEC_PART_ARGS);
@@ -322,13 +286,13 @@ __global__ __launch_bounds__(128) void attn_decode_combine_kernel(
     const float* pm = part_ml + ((size_t)di * Hq + head) * max_splits * 2;
     const float* pa = part_acc + ((size_t)di * Hq + head) * max_splits * D;
     if (tid < 64) {                                    // first wave: maximum, weights, sum in split order
-        float m = -INFINITY;
+        float m = -INFINITY;                           // (the maxima are base-2 exponents)
         for (int s = tid; s < ns; s += 64) m = fmaxf(m, pm[2 * s]);
         m = wave_max(m);
-        for (int s = tid; s < ns; s += 64) w_s[s] = __expf(pm[2 * s] - m);
+        for (int s = tid; s < ns; s += 64) w_s[s] = __builtin_amdgcn_exp2f(pm[2 * s] - m);
         if (tid == 0) {
             float l = 0.f;
-            for (int s = 0; s < ns; ++s) l += pm[2 * s + 1] * __expf(pm[2 * s] - m);
+            for (int s = 0; s < ns; ++s) l += pm[2 * s + 1] * __builtin_amdgcn_exp2f(pm[2 * s] - m);
             stat[0] = l > 0.f ? 1.0f / l : 0.f;
         }
     }
@@ -359,10 +323,6 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(n_dec, Hkv, max_splits);
-    const int G = Hq / Hkv;
-    const int kpi = 64 / (D / 8);
-    const size_t shmem = (size_t)kpi * G * D * sizeof(float);
-    if (shmem > 48 * 1024) return RA_ERR_ARG;
     const bf16* qq = (const bf16*)q;
     const bf16* kp = (const bf16*)k_pool;
     const bf16* vp = (const bf16*)v_pool;
@@ -371,10 +331,10 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
     int rc;
     const int d16 = D / 16;
     switch ((d16 - 1) / 4) {
-        case 0: rc = ra_dec_part_0(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        case 1: rc = ra_dec_part_1(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        case 2: rc = ra_dec_part_2(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        case 3: rc = ra_dec_part_3(d16, G, grid, shmem, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 0: rc = ra_dec_part_0(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 1: rc = ra_dec_part_1(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 2: rc = ra_dec_part_2(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
+        case 3: rc = ra_dec_part_3(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
         default: return RA_ERR_ARG;
     }
     if (rc != RA_OK) return rc;
