@@ -386,6 +386,118 @@ __global__ void qkv_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, i
     }
 }
 
+// The same for bfloat16 with 16-byte accesses, when the whole head rotates (R == D) or nothing
+// does (R == 0) and D % 16 == 0: a group of GP lanes (a power of two >= D/16) takes one
+// (token, head); a lane holds eight elements of the first half and their eight partners of the
+// second half, so a rotary pair never leaves its lane.
+typedef uint32_t qkv_u4 __attribute__((ext_vector_type(4)));
+typedef float qkv_f4 __attribute__((ext_vector_type(4)));
+template <int GP>
+__global__ __launch_bounds__(256) void qkv_prepare_bf16x8_kernel(
+    const bf16* __restrict__ qkv, int Hq, int Hkv, int D, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, const int* __restrict__ positions,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int R, bf16* __restrict__ q_out,
+    bf16* __restrict__ k_pool, bf16* __restrict__ v_pool, const int* __restrict__ slots,
+    long long pool_rows, long long n_rows) {
+    const long long row = ((long long)blockIdx.x * 256 + threadIdx.x) / GP;      // (token, head)
+    const int sub = threadIdx.x % GP;
+    const int half = D >> 1;
+    const int j0 = sub * 8;
+    const int heads = Hq + 2 * Hkv;
+    const bool in = row < n_rows && j0 < half;
+    const int t = in ? (int)(row / heads) : 0;
+    const int head = in ? (int)(row % heads) : 0;
+    const bf16* src = qkv + (in ? row : 0) * D;
+
+    bf16* dst = nullptr;
+    const float* w = nullptr;
+    bool rotate = false;
+    if (in) {
+        if (head < Hq) {
+            dst = q_out + ((size_t)t * Hq + head) * D;
+            w = wq;
+            rotate = R > 0;
+        } else {
+            const int kvh = (head - Hq) % Hkv;
+            const bool is_k = head < Hq + Hkv;
+            bf16* pool = is_k ? k_pool : v_pool;
+            const long long s = slots[t];
+            if (pool != nullptr && s >= 0 && s < pool_rows) dst = pool + ((size_t)s * Hkv + kvh) * D;
+            if (is_k) {
+                w = wk;
+                rotate = R > 0;
+            }
+        }
+    }
+    float a[8], b[8];
+    if (in) {
+        const qkv_u4 a4 = *reinterpret_cast<const qkv_u4*>(src + j0);
+        const qkv_u4 b4 = *reinterpret_cast<const qkv_u4*>(src + half + j0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[2 * i] = __uint_as_float(a4[i] << 16);
+            a[2 * i + 1] = __uint_as_float(a4[i] & 0xffff0000u);
+            b[2 * i] = __uint_as_float(b4[i] << 16);
+            b[2 * i + 1] = __uint_as_float(b4[i] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = b[i] = 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += a[i] * a[i] + b[i] * b[i];
+#pragma unroll
+    for (int o = GP / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);      // every lane of the wave takes part
+    if (dst == nullptr) return;
+    if (w != nullptr) {
+        const float rstd = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const qkv_f4 w1 = *reinterpret_cast<const qkv_f4*>(w + j0 + 4 * i);
+            const qkv_f4 w2 = *reinterpret_cast<const qkv_f4*>(w + half + j0 + 4 * i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a[4 * i + e] = a[4 * i + e] * rstd * w1[e];
+                b[4 * i + e] = b[4 * i + e] * rstd * w2[e];
+            }
+        }
+    }
+    if (rotate) {
+        const size_t at = (size_t)positions[t] * half + j0;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const qkv_f4 c4 = *reinterpret_cast<const qkv_f4*>(cos_t + at + 4 * i);
+            const qkv_f4 s4 = *reinterpret_cast<const qkv_f4*>(sin_t + at + 4 * i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float x1 = a[4 * i + e], x2 = b[4 * i + e];
+                a[4 * i + e] = x1 * c4[e] - x2 * s4[e];
+                b[4 * i + e] = x2 * c4[e] + x1 * s4[e];
+            }
+        }
+    }
+    qkv_u4 oa, ob;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        oa[i] = (uint32_t)f2bf_bits(a[2 * i]) | ((uint32_t)f2bf_bits(a[2 * i + 1]) << 16);
+        ob[i] = (uint32_t)f2bf_bits(b[2 * i]) | ((uint32_t)f2bf_bits(b[2 * i + 1]) << 16);
+    }
+    *reinterpret_cast<qkv_u4*>(dst + j0) = oa;
+    *reinterpret_cast<qkv_u4*>(dst + half + j0) = ob;
+}
+
+template <int GP>
+static void launch_qkv_prepare_x8(long long n_rows, hipStream_t st, const bf16* qkv, int Hq, int Hkv, int D,
+                                  const float* wq, const float* wk, float eps, const int* positions,
+                                  const float* cos_t, const float* sin_t, int R, bf16* q_out, bf16* k_pool,
+                                  bf16* v_pool, const int* slots, long long pool_rows) {
+    const long long threads = n_rows * GP;
+    hipLaunchKernelGGL(qkv_prepare_bf16x8_kernel<GP>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                       st, qkv, Hq, Hkv, D, wq, wk, eps, positions, cos_t, sin_t, R, q_out, k_pool, v_pool,
+                       slots, pool_rows, n_rows);
+}
+
 extern "C" int ra_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, int D, const float* wq,
                               const float* wk, float eps, const int* positions, const float* cos_t,
                               const float* sin_t, int R, void* q_out, void* k_pool, void* v_pool,
@@ -395,6 +507,21 @@ extern "C" int ra_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, in
     // pairs: R/2 <= 256; pass-through: D-R <= 256
     if ((R >> 1) > 64 * QKV_MAX_PER_LANE || (D - R) > 64 * QKV_MAX_PER_LANE) return RA_ERR_ARG;
     const long long n_rows = (long long)T_tokens * (Hq + 2 * Hkv);
+    if (dtype == RA_DTYPE_BF16 && D % 16 == 0 && (R == D || R == 0) && n_rows * 32 < (1ll << 31) * 256) {
+        const int lanes = D / 16;                 // lanes that a head needs
+#define QKV_X8(GP)                                                                                    \
+    launch_qkv_prepare_x8<GP>(n_rows, (hipStream_t)stream, (const bf16*)qkv, Hq, Hkv, D, wq, wk, eps,  \
+                              positions, cos_t, sin_t, R, (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool,  \
+                              slots, pool_rows)
+        if (lanes <= 1) QKV_X8(1);
+        else if (lanes <= 2) QKV_X8(2);
+        else if (lanes <= 4) QKV_X8(4);
+        else if (lanes <= 8) QKV_X8(8);
+        else if (lanes <= 16) QKV_X8(16);
+        else QKV_X8(32);
+#undef QKV_X8
+        return ra_launch_status();
+    }
     dim3 block(256), grid((unsigned)((n_rows + 3) / 4));
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(qkv_prepare_kernel<float>, grid, block, 0, (hipStream_t)stream,

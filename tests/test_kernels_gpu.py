@@ -102,7 +102,9 @@ def test_head_rmsnorm_and_rope(ops, ref, dtype, D):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,D,R,norm", [(4, 2, 16, 16, True), (6, 1, 32, 32, True), (5, 5, 48, 48, True),
                                            (3, 1, 80, 32, False), (8, 2, 128, 128, True),
-                                           (2, 2, 256, 64, True), (1, 1, 512, 512, True)])
+                                           (2, 2, 256, 64, True), (1, 1, 512, 512, True),
+                                           (7, 1, 80, 80, True), (2, 1, 192, 192, False), (3, 1, 64, 0, True),
+                                           (9, 3, 256, 256, True)])
 def test_qkv_prepare(ops, ref, dtype, Hq, Hkv, D, R, norm):
     T, P, pages = 11, 8, 6
     qkv = rnd(T, (Hq + 2 * Hkv) * D, dtype=dtype, seed=11)
