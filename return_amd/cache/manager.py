@@ -62,9 +62,12 @@ class PagedGroup:
         self.num_pages = num_pages
         self.page_size = page_size
         # [layer, k|v, page, row in page, kv head, D]: one token-head row is contiguous,
-        # a page of one layer is one contiguous run of P*Hkv*D elements.
-        self.pool = torch.zeros(len(self.layers), 2, num_pages, page_size, spec.num_kv_heads,
+        # a page of one layer is one contiguous run of P*Hkv*D elements. One page beyond the
+        # num_pages that requests can hold is the spare page: rows that only fill a batch up
+        # to a fixed size (pad_tables) write and read there.
+        self.pool = torch.zeros(len(self.layers), 2, num_pages + 1, page_size, spec.num_kv_heads,
                                 spec.head_dim, dtype=dtype, device=device)
+        self.spare_page = num_pages
         self.pages = FreeList(num_pages, "page")
 
     def layer_pools(self, cache_layer: int) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -121,10 +124,11 @@ class CacheManager:
                                          for layer in grp.layers}
 
         self.slots = FreeList(self.max_requests, "request slot")
+        self.spare_slot = self.max_requests      # the state row of rows that only fill a batch up
         self.state: Dict[int, Dict[str, torch.Tensor]] = {}
         for layer, spec in self.state_layers.items():
             self.state[layer] = {
-                name: torch.zeros((self.max_requests,) + tuple(shape), dtype=_DTYPES[dt], device=device)
+                name: torch.zeros((self.max_requests + 1,) + tuple(shape), dtype=_DTYPES[dt], device=device)
                 for name, shape, dt in spec.tensors}
 
         self.live: Dict[object, _Live] = {}
@@ -264,6 +268,31 @@ class CacheManager:
         return StepTables([rid for rid, _ in entries], q_lens, q_start, cu_q, positions,
                           seq_lens, slot_ids, groups)
 
+    def pad_tables(self, tables: StepTables, n_pad: int) -> StepTables:
+        """The same step with n_pad more one-token sequences that belong to no request: token
+        at position 0, written to and read from the spare page (state: the spare slot). A
+        decode step of a few fixed sizes can be replayed from a few captured graphs; what the
+        added rows compute is thrown away and touches nothing that a request holds."""
+        if n_pad <= 0:
+            return tables
+        P = self.page_size
+        one = np.ones(n_pad, dtype=np.int32)
+        last = int(tables.cu_q[-1])
+        groups = []
+        for grp, gt in zip(self.groups, tables.groups):
+            groups.append(GroupTables(
+                np.concatenate([gt.slot_mapping, one * (grp.spare_page * P)]).astype(np.int32),
+                np.concatenate([gt.page_table, one * grp.spare_page]).astype(np.int32),
+                np.concatenate([gt.cu_pages, gt.cu_pages[-1] + np.arange(1, n_pad + 1)]).astype(np.int32),
+                np.concatenate([gt.kv_start, 0 * one]).astype(np.int32)))
+        return StepTables(
+            list(tables.request_ids) + [None] * n_pad, list(tables.q_lens) + [1] * n_pad,
+            np.concatenate([tables.q_start, 0 * one]).astype(np.int32),
+            np.concatenate([tables.cu_q, last + np.arange(1, n_pad + 1)]).astype(np.int32),
+            np.concatenate([tables.positions, 0 * one]).astype(np.int32),
+            np.concatenate([tables.seq_lens, one]).astype(np.int32),
+            np.concatenate([tables.slot_ids, one * self.spare_slot]).astype(np.int32), groups)
+
     def end_step(self) -> None:
         """After the step ran: give back pages that every later query's window has passed."""
         P = self.page_size
@@ -333,4 +362,4 @@ class PagedView:
 
 @dataclasses.dataclass
 class StateView:
-    tensors: Dict[str, torch.Tensor]    # name -> [max_requests, ...]; row = StepBatch.slot_ids
+    tensors: Dict[str, torch.Tensor]    # name -> [max_requests + 1, ...]; row = StepBatch.slot_ids

@@ -58,7 +58,7 @@ def cmd_generate(args) -> int:
     parsed = [parse_request(r, i) for i, r in enumerate(raws)]
     engine = Engine(args.model, max_token=args.max_token, max_reside=args.max_reside, dtype=args.dtype,
                     page_size=args.page_size, seed=args.seed, max_step_tokens=args.max_step_tokens,
-                    prefill_chunk=args.prefill_chunk)
+                    prefill_chunk=args.prefill_chunk, use_graphs=not args.no_graphs)
     results = engine.generate([p for _, p, _ in parsed], [sp for _, _, sp in parsed])
     for (sid, _, _), r in zip(parsed, results):
         out = {"session_id": sid, "output_ids": r.output_ids, "output_logprobs": r.output_logprobs,
@@ -95,6 +95,8 @@ def main(argv=None) -> int:
     g.add_argument("--max-step-tokens", type=int, default=8192)
     g.add_argument("--prefill-chunk", type=int, default=8192)
     g.add_argument("--seed", type=int, default=0)
+    g.add_argument("--no-graphs", action="store_true",
+                   help="launch every kernel of a decode step from the host instead of replaying HIP graphs")
     g.add_argument("--requests", help="file of JSON lines (or - for standard input), one request each")
     g.add_argument("--prompt-ids", help="one prompt as comma-separated token ids")
     g.add_argument("--max-new-tokens", type=int, default=32)

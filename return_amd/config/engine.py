@@ -18,7 +18,7 @@ class EngineConfig:
     max_reside: int = 64               # most requests that are live at a time
     max_step_tokens: int = 8192        # token budget of one step (decoded tokens + prompt portions)
     prefill_chunk: int = 8192          # longest portion of one prompt in one step
-    use_graphs: bool = False           # replay decode-only steps from captured HIP graphs
+    use_graphs: bool = True            # replay decode-only steps from captured HIP graphs (USE_CUDA_GRAPH of the reference)
     seed: int = 0                      # base seed of the sampling streams
     device: str = "cuda:0"
 

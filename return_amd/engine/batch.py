@@ -99,9 +99,10 @@ class StepBuilder:
             self._off[name] = (off, size)
             off += -(-size // 4) * 4          # keep every table 16-byte aligned
         self._small_end = off
-        # a windowed request lists at most its held pages; the sum over a step never exceeds the pool
+        # a windowed request lists at most its held pages; the sum over a step never exceeds the
+        # pool, plus the spare page once for every row that only fills the batch up
         for g in range(G):
-            size = cache.groups[g].num_pages
+            size = cache.groups[g].num_pages + N
             self._off[f"page_table{g}"] = (off, size)
             off += -(-size // 4) * 4
         self._total = off

@@ -147,19 +147,33 @@ class ModelRunner:
                 raise ValueError(f"request {rid!r}: token {t} outside the vocabulary of {self.vocab_size}")
             if self.cache.seq_len(rid) + 1 > self.max_position:
                 raise ValueError(f"request {rid!r} would pass max_position_embeddings {self.max_position}")
+        graphs = self.engine_config.use_graphs and self.rt.device.type == "cuda"
+        rows = self.graph_batch_size(n) if graphs else n
+        pad = rows - n
         tables = self.cache.begin_step([(rid, 1) for rid in request_ids])
         try:
-            batch = self.builder.build(tables, [[int(t)] for t in tokens], list(range(n)))
-            self._put_sampling(n, temperature, top_k, top_p, uniforms)
+            tables = self.cache.pad_tables(tables, pad)
+            batch = self.builder.build(tables, [[int(t)] for t in tokens] + [[0]] * pad, list(range(rows)))
+            # rows that only fill the batch up are chosen greedily and thrown away
+            self._put_sampling(rows, list(temperature) + [0.0] * pad, list(top_k) + [0] * pad,
+                               list(top_p) + [1.0] * pad, list(uniforms) + [0.0] * pad)
             with torch.no_grad():
-                if self.engine_config.use_graphs and self.rt.device.type == "cuda":
+                if graphs:
                     logits, picked = self._replay(batch)
                 else:
                     logits, picked = self._decode_body(batch)
         finally:
             self.cache.end_step()
-        host = picked.cpu()
-        return host[:, 0].tolist(), host[:, 1].contiguous().view(torch.float32).tolist(), logits
+        host = picked[:n].cpu()
+        return host[:, 0].tolist(), host[:, 1].contiguous().view(torch.float32).tolist(), logits[:n]
+
+    def graph_batch_size(self, n: int) -> int:
+        """The batch size whose graph serves n decoding requests: n itself up to 8, then the
+        next multiple of 8 (never more than max_reside), so that a batch that shrinks one
+        request at a time does not capture a graph per size."""
+        if n <= 8:
+            return n
+        return min(-(-n // 8) * 8, max(n, self.engine_config.max_reside))
 
     def _replay(self, batch):
         bucket = 256

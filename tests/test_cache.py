@@ -157,7 +157,8 @@ def test_state_slots():
     cm = manager(extra={5: spec}, max_requests=2)
     s0 = cm.add_request("a")
     view = cm.view(5)
-    assert view.tensors["rec"].shape == (2, 2, 4, 4) and view.tensors["conv"].dtype == torch.bfloat16
+    assert view.tensors["rec"].shape == (2 + 1, 2, 4, 4)       # one row per slot and the spare row
+    assert view.tensors["conv"].dtype == torch.bfloat16
     view.tensors["rec"][s0] += 3.0
     cm.add_request("b")
     with pytest.raises(KVCapacityError):
@@ -189,4 +190,36 @@ def test_groups_have_pools_of_their_own():
     assert sorted(map(tuple, (g.layers for g in cm.groups))) == [(0, 3), (1,), (2,)]
     v0, v3 = cm.view(0), cm.view(3)
     assert v0.group == v3.group and v0.k_pool.data_ptr() != v3.k_pool.data_ptr()
-    assert v0.k_pool.shape == (8, 4, 2, 8) and cm.view(2).k_pool.shape == (8, 4, 1, 16)
+    # 32 tokens in pages of 4, and the spare page
+    assert v0.k_pool.shape == (8 + 1, 4, 2, 8) and cm.view(2).k_pool.shape == (8 + 1, 4, 1, 16)
+
+
+def test_pad_tables_adds_rows_on_the_spare_page_only():
+    """Rows that fill a batch up belong to no request: they sit at position 0 of the spare page
+    and of the spare state slot, and change nothing the manager keeps."""
+    from return_amd.cache import StateSpec
+    cm = CacheManager({0: PagedKVSpec(2, 8, None), 1: PagedKVSpec(1, 8, 4), 2: StateSpec((("s", (3,), "float32"),))},
+                      page_size=4, max_token=64, max_requests=3, dtype=torch.float32)
+    cm.add_request("a"); cm.add_request("b")
+    cm.begin_step([("a", 6), ("b", 3)]); cm.end_step()
+    t = cm.begin_step([("a", 1), ("b", 1)])
+    before = (cm.free_pages(), cm.free_slots(), {k: (v.seq_len, [list(p) for p in v.pages]) for k, v in cm.live.items()})
+    p = cm.pad_tables(t, 3)
+    after = (cm.free_pages(), cm.free_slots(), {k: (v.seq_len, [list(p) for p in v.pages]) for k, v in cm.live.items()})
+    assert before == after
+    assert cm.pad_tables(t, 0) is t
+    assert p.request_ids == ["a", "b", None, None, None] and p.q_lens == [1, 1, 1, 1, 1]
+    assert p.cu_q.tolist() == [0, 1, 2, 3, 4, 5]
+    assert p.positions.tolist() == t.positions.tolist() + [0, 0, 0]
+    assert p.q_start.tolist()[2:] == [0, 0, 0] and p.seq_lens.tolist()[2:] == [1, 1, 1]
+    assert p.slot_ids.tolist()[2:] == [cm.spare_slot] * 3 and cm.spare_slot == 3
+    for grp, g0, g1 in zip(cm.groups, t.groups, p.groups):
+        assert grp.spare_page == grp.num_pages and grp.pool.shape[2] == grp.num_pages + 1
+        assert g1.slot_mapping.tolist() == g0.slot_mapping.tolist() + [grp.spare_page * 4] * 3
+        assert g1.page_table.tolist() == g0.page_table.tolist() + [grp.spare_page] * 3
+        assert g1.cu_pages.tolist() == g0.cu_pages.tolist() + [g0.cu_pages[-1] + i for i in (1, 2, 3)]
+        assert g1.kv_start.tolist()[2:] == [0, 0, 0]
+        assert grp.spare_page not in grp.pages.free_ids()
+    assert cm.state[2]["s"].shape[0] == 4
+    cm.end_step()
+    cm.check_invariants()

@@ -49,6 +49,44 @@ def test_graph_replays_match_eager(folder_b, dtype):
     assert te == tg and torch.equal(logits_e, logits_g)
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_batch_filled_up_to_a_graph_size(folder_b, dtype):
+    """Eleven requests run from the graph of sixteen: the five added rows write and read the
+    spare page only; logits, tokens and every page that a request holds equal the eager run."""
+    V = TINY_B["vocab_size"]
+    lens = [5, 17, 33, 64, 2, 90, 16, 47, 1, 129, 31]
+
+    def make(use_graphs):
+        ec = EngineConfig(dtype=dtype, page_size=16, max_token=4096, max_reside=16, max_step_tokens=512,
+                          prefill_chunk=512, use_graphs=use_graphs)
+        r = ModelRunner(folder_b, engine_config=ec)
+        for i, n in enumerate(lens):
+            r.add_request(i)
+            r.step([StepEntry(i, tt.random_tokens(V, n, seed=100 + n), [])])
+        return r
+
+    eager, graph = make(False), make(True)
+    assert graph.graph_batch_size(11) == 16 and graph.graph_batch_size(8) == 8 and graph.graph_batch_size(16) == 16
+    ids = list(range(len(lens)))
+    toks = [3 + i for i in ids]
+    zeros, ones = [0.0] * len(ids), [1.0] * len(ids)
+    for step in range(20):
+        te, le, logits_e = eager.decode_and_sample(ids, toks, zeros, [0] * len(ids), ones, zeros)
+        tg, lg, logits_g = graph.decode_and_sample(ids, toks, zeros, [0] * len(ids), ones, zeros)
+        assert logits_g.shape == logits_e.shape and torch.equal(logits_e, logits_g), f"step {step}"
+        assert te == tg and le == lg
+        toks = te
+        if step == 9:                               # the batch shrinks: ten requests, the same graph size
+            for r in (eager, graph):
+                r.free_request(ids[-1])
+            ids, toks = ids[:-1], toks[:-1]
+            zeros, ones = zeros[:-1], ones[:-1]
+    assert {k[0] for k in graph._graphs} == {16}
+    for ge, gg in zip(eager.cache.groups, graph.cache.groups):
+        assert torch.equal(ge.pool[:, :, :ge.num_pages], gg.pool[:, :, :gg.num_pages])
+    graph.cache.check_invariants()
+
+
 def test_generation_with_graphs(folder_b):
     from return_amd import SamplingParams
     from return_amd.engine import Engine
