@@ -178,8 +178,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
                 mx = fmaxf(mx, s[st][i]);
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = rows_max(mx);
         const float m_new = fmaxf(m_run, mx);            // finite: the pass holds a valid key
         float lsum = 0.f;
 #pragma unroll
@@ -189,8 +188,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
                 s[st][i] = __builtin_amdgcn_exp2f(s[st][i] - m_new);   // 2^(-inf) = 0 for masked keys
                 lsum += s[st][i];
             }
-        lsum += __shfl_xor(lsum, 16, 64);
-        lsum += __shfl_xor(lsum, 32, 64);
+        lsum = rows_sum(lsum);
         const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
         l_run = l_run * alpha + lsum;
         if (__any(m_new != m_run)) {

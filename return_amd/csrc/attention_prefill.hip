@@ -10,11 +10,14 @@
 //
 // BUILD-VARIANTS: PRE_PART=0 PRE_PART=1 PRE_PART=2 PRE_PART=3 PRE_API=1
 //
-// One workgroup of four waves per (q tile of 64 rows, query head); wave w owns rows 16w..16w+15.
+// One workgroup of four waves per (q tile of 64*QG rows, query head); wave w owns QG groups of
+// 16 rows, 16*QG*w .. 16*QG*(w+1)-1. QG is 2 up to head size 128 and 1 beyond: with two groups
+// every operand that comes out of LDS (a K row piece, a V^T piece) feeds two MFMAs, which
+// halves the LDS traffic per flop; beyond 128 the accumulators of two groups no longer fit.
 // Per pass a tile of BN keys sits in LDS, K and V both row-major with padded rows; the next
 // tile's rows are already on their way from the cache into registers while this one is used.
-//  scores  S^T = K Q^T by MFMA 16x16x32 bf16: A = K tile rows from LDS, B = the wave's 16
-//          query rows held in registers. Lane (n, g) gets query n, keys 4g..4g+3 of each
+//  scores  S^T = K Q^T by MFMA 16x16x32 bf16: A = K tile rows from LDS, B = 16 query rows
+//          held in registers. Lane (n, g) gets query n of each group, keys 4g..4g+3 of each
 //          16-key tile.
 //  P.V     O^T += V^T P^T by the same MFMA. The contraction runs over keys in the order the
 //          lanes already hold them: k-slot (g, e) of a 32-key block is key 16*(e/4) + 4g + e%4,
@@ -31,7 +34,8 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-#define PRE_BM 64
+// head sizes up to 16 * PRE_WIDE_D16 run two groups of query rows per wave (tiles of 128 rows)
+#define PRE_WIDE_D16 8
 
 #ifdef PRE_PART
 
@@ -48,8 +52,8 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 typedef short4_t __attribute__((address_space(3))) * lds_short4_ptr;
 
-template <int D16>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+template <int D16, int QG, int KSPLIT>
+__global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ page_table,
     const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
@@ -59,6 +63,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;
     constexpr bool TAIL16 = (D % 32) != 0;
+    constexpr int BM = 64 * QG;                         // query rows per workgroup
     constexpr int BN = (D <= 128) ? 64 : 32;            // keys per pass
     constexpr int KS = D + 8;                           // K tile row stride (elements): rows shift by 4 banks
     constexpr int VS = D + 16;                          // V tile row stride: rows shift by 8 banks (transposing reads)
@@ -66,9 +71,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     constexpr int TPK = 256 / BN;                       // threads that share the loading of one key row
     constexpr int NLD = (LPR + TPK - 1) / TPK;          // pieces of K (and of V) per thread per tile
 
-    // two tiles: one is used while the next is written
-    __shared__ __attribute__((aligned(16))) uint16_t k_s[2][BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t v_s[2][BN * VS];
+    // Per group of four waves two tiles of K and of V: one is used while the next is written. With
+    // KSPLIT == 2 a second group of four waves works on the same query rows and takes every other
+    // key tile; at the end its sums are merged into the first group's through the same memory.
+    constexpr int TILE = BN * KS + BN * VS;             // elements of one K tile and one V tile
+    constexpr int MERGE_SLOTS = 4 * D16 + 2;            // per lane and query group: the accumulators, m and l
+    constexpr size_t TILE_BYTES = (size_t)KSPLIT * 2 * TILE * 2;
+    constexpr size_t MERGE_BYTES = KSPLIT > 1 ? (size_t)4 * QG * MERGE_SLOTS * 64 * 4 : 0;
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES];
+    const int grp = threadIdx.x >> 8;                   // which group of four waves
+    uint16_t* const tiles_s = reinterpret_cast<uint16_t*>(lds_raw) + (size_t)grp * 2 * TILE;
+#define K_S(buf_) (tiles_s + (buf_) * TILE)
+#define V_S(buf_) (tiles_s + (buf_) * TILE + BN * KS)
 
     // Workgroups go to the 8 XCDs round-robin by their number, and each XCD has an L2 of its own:
     // all workgroups of one kv head are sent to the same XCD, so that its keys and values are
@@ -90,46 +104,55 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         }
     }
     const int seg = tiles[2 * tile], q_off = tiles[2 * tile + 1];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x & 255, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int kvh = head / (Hq / Hkv);
     const int q_len = cu_q[seg + 1] - cu_q[seg];
     const int pos0 = q_start[seg];                       // position of the request's first new token
     const int start = kv_start[seg];
     const int* pt = page_table + cu_pages[seg];
 
-    // this lane's query row (for the B operand and for the mask): row n of the wave's 16
-    const int q_local = q_off + wave * 16 + n;
-    const bool q_ok = q_local < q_len;
-    const int pos_q = pos0 + q_local;
+    // this lane's query rows (for the B operands and for the mask): row n of each of the wave's groups
+    int pos_q[QG];
+    bool q_ok[QG];
     const bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8_t bq[D32 > 0 ? D32 : 1];
-    bf16x8_t bq_tail = z8;
-    {
-        const bf16* qp = q + ((size_t)(cu_q[seg] + (q_ok ? q_local : 0)) * Hq + head) * D;
+    bf16x8_t bq[QG][D32 > 0 ? D32 : 1];
+    bf16x8_t bq_tail[QG];
+#pragma unroll
+    for (int qg = 0; qg < QG; ++qg) {
+        const int q_local = q_off + (wave * QG + qg) * 16 + n;
+        q_ok[qg] = q_local < q_len;
+        pos_q[qg] = pos0 + q_local;
+        const bf16* qp = q + ((size_t)(cu_q[seg] + (q_ok[qg] ? q_local : 0)) * Hq + head) * D;
 #pragma unroll
         for (int j = 0; j < D32; ++j) {
             bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(qp + 32 * j + 8 * g);
-            bq[j] = q_ok ? v : z8;
+            bq[qg][j] = q_ok[qg] ? v : z8;
         }
+        bq_tail[qg] = z8;
         if constexpr (TAIL16) {
-            if (q_ok && g < 2) bq_tail = *reinterpret_cast<const bf16x8_t*>(qp + (D - 16) + 8 * g);
+            if (q_ok[qg] && g < 2) bq_tail[qg] = *reinterpret_cast<const bf16x8_t*>(qp + (D - 16) + 8 * g);
         }
     }
 
     // keys this tile needs: from the earliest key any of its rows may read to its last row's position
     const int tile_first_pos = pos0 + q_off;
-    const int tile_last_pos = pos0 + min(q_off + PRE_BM, q_len) - 1;
+    const int tile_last_pos = pos0 + min(q_off + BM, q_len) - 1;
     int first_key = start;
     if (window > 0 && tile_first_pos - window + 1 > first_key) first_key = tile_first_pos - window + 1;
 
     const float scale2 = scale * 1.44269504088896340736f;
     // positions of the first and last row of this wave (wave-uniform, for skipping the mask)
-    const int wave_first_pos = pos0 + q_off + wave * 16;
-    const int wave_last_pos = wave_first_pos + 15;
-    float m_run = -INFINITY, l_run = 0.f;
-    float4_t acc[D16];
+    const int wave_first_pos = pos0 + q_off + wave * QG * 16;
+    const int wave_last_pos = wave_first_pos + QG * 16 - 1;
+    float m_run[QG], l_run[QG];
+    float4_t acc[QG][D16];
 #pragma unroll
-    for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int qg = 0; qg < QG; ++qg) {
+        m_run[qg] = -INFINITY;
+        l_run[qg] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < D16; ++dt) acc[qg][dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     // what each thread moves per tile: its key row's pieces my_sub, my_sub + TPK, ... of K and of V
     uint4_t kreg[NLD], vreg[NLD];                        // native vectors: they stay in registers
@@ -157,118 +180,131 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                               \
         const int p_ = my_sub + TPK * i;                                            \
         if (p_ < LPR) {                                                             \
-            *reinterpret_cast<uint4_t*>(&k_s[buf_][my_key * KS + 8 * p_]) = kreg[i]; \
-            *reinterpret_cast<uint4_t*>(&v_s[buf_][my_key * VS + 8 * p_]) = vreg[i]; \
+            *reinterpret_cast<uint4_t*>(K_S(buf_) + my_key * KS + 8 * p_) = kreg[i]; \
+            *reinterpret_cast<uint4_t*>(V_S(buf_) + my_key * VS + 8 * p_) = vreg[i]; \
         }                                                                           \
     }
+    // group grp takes the key tiles grp, grp + KSPLIT, grp + 2 KSPLIT, ... counted from c_first
     const int c_first = (first_key / BN) * BN;
+    constexpr int STEP = KSPLIT * BN;                    // from one tile of a group to its next
     int row_next;                                        // row of this thread's key in the tile fetched next
     {
-        const int r0 = ROW_OF(c_first + my_key);
-        row_next = ROW_OF(c_first + BN + my_key);
+        const int c_mine = c_first + grp * BN;
+        const int r0 = ROW_OF(c_mine + my_key);
+        row_next = ROW_OF(c_mine + STEP + my_key);
         FETCH_ROW(r0)
         STAGE_TO(0)
-        FETCH_ROW(row_next)                              // tile 1 (or a repeat of valid rows if there is none)
-        row_next = ROW_OF(c_first + 2 * BN + my_key);
+        FETCH_ROW(row_next)                              // the group's second tile (or a repeat of valid rows if there is none)
+        row_next = ROW_OF(c_mine + 2 * STEP + my_key);
     }
     __syncthreads();
 
     int it = 0;
-    for (int c0 = c_first; c0 <= tile_last_pos; c0 += BN, ++it) {
+    for (int c_it = c_first; c_it <= tile_last_pos; c_it += STEP, ++it) {
+        const int c0 = c_it + grp * BN;                  // beyond tile_last_pos: this group sits the pass out
         const int cur = it & 1;
-        const uint16_t* k_cur = k_s[cur];
-        const uint16_t* v_cur = v_s[cur];
-        if (c0 + BN <= tile_last_pos) {
+        const uint16_t* k_cur = K_S(cur);
+        const uint16_t* v_cur = V_S(cur);
+        if (c0 + STEP <= tile_last_pos) {
             // the next tile, asked for one pass ago, goes into the other buffer (which every wave left
             // at the last barrier); then the tile after it is asked for
             STAGE_TO(cur ^ 1)
-            if (c0 + 2 * BN <= tile_last_pos) {
+            if (c0 + 2 * STEP <= tile_last_pos) {
                 FETCH_ROW(row_next)
-                row_next = ROW_OF(c0 + 3 * BN + my_key);
+                row_next = ROW_OF(c0 + 3 * STEP + my_key);
             }
         }
 
-        // ---- scores of the wave's 16 rows against the BN keys
-        float4_t cs[BN / 16];
+        // a tile that lies wholly above every row of the wave has nothing for it
+        if (c0 <= wave_last_pos && c0 <= tile_last_pos) {
+        // ---- scores of the wave's rows against the BN keys; a K piece from LDS serves every group
+        float4_t cs[QG][BN / 16];
 #pragma unroll
         for (int st = 0; st < BN / 16; ++st) {
-            float4_t c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int qg = 0; qg < QG; ++qg) cs[qg][st] = float4_t{0.f, 0.f, 0.f, 0.f};
             const uint16_t* kr = &k_cur[(st * 16 + n) * KS];
 #pragma unroll
             for (int j = 0; j < D32; ++j) {
                 const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(kr + 32 * j + 8 * g);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[j], c, 0, 0, 0);
+#pragma unroll
+                for (int qg = 0; qg < QG; ++qg)
+                    cs[qg][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[qg][j], cs[qg][st], 0, 0, 0);
             }
             if constexpr (TAIL16) {
                 bf16x8_t a = z8;
                 if (g < 2) a = *reinterpret_cast<const bf16x8_t*>(kr + (D - 16) + 8 * g);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq_tail, c, 0, 0, 0);
+#pragma unroll
+                for (int qg = 0; qg < QG; ++qg)
+                    cs[qg][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq_tail[qg], cs[qg][st], 0, 0, 0);
             }
-            cs[st] = c;
         }
         MFMA_SETTLE();
         // Scores in the base-2 domain: s2 = (q.k) * scale * log2(e), so that p = 2^(s2 - m).
-        float s[BN / 16][4];
-        float mx = -INFINITY;
         // a tile that lies wholly below every row of the wave and inside every window needs no mask
         const bool need_mask = (c0 + BN - 1 > wave_first_pos) || (c0 < first_key) ||
                                (window > 0 && c0 <= wave_last_pos - window);
-        if (need_mask) {
+        uint4_t pw[QG][BN / 32];                         // P as bf16, in the order the B operand wants
 #pragma unroll
-            for (int st = 0; st < BN / 16; ++st) {
+        for (int qg = 0; qg < QG; ++qg) {
+            float s[BN / 16][4];
+            float mx = -INFINITY;
+            if (need_mask) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int kpos = c0 + st * 16 + 4 * g + i;
-                    bool ok = kpos >= first_key && kpos <= pos_q;
-                    if (window > 0) ok = ok && kpos > pos_q - window;
-                    s[st][i] = ok ? cs[st][i] * scale2 : -INFINITY;
-                    mx = fmaxf(mx, s[st][i]);
+                for (int st = 0; st < BN / 16; ++st) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int kpos = c0 + st * 16 + 4 * g + i;
+                        bool ok = kpos >= first_key && kpos <= pos_q[qg];
+                        if (window > 0) ok = ok && kpos > pos_q[qg] - window;
+                        s[st][i] = ok ? cs[qg][st][i] * scale2 : -INFINITY;
+                        mx = fmaxf(mx, s[st][i]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int st = 0; st < BN / 16; ++st) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        s[st][i] = cs[qg][st][i] * scale2;
+                        mx = fmaxf(mx, s[st][i]);
+                    }
                 }
             }
-        } else {
+            mx = rows_max(mx);
+            const float m_new = fmaxf(m_run[qg], mx);
+            // a row that sees no key yet (all of this pass lies above it or outside its window) keeps m = -inf
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float lsum = 0.f;
 #pragma unroll
-            for (int st = 0; st < BN / 16; ++st) {
+            for (int st = 0; st < BN / 16; ++st)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    s[st][i] = cs[st][i] * scale2;
-                    mx = fmaxf(mx, s[st][i]);
+                    s[st][i] = __builtin_amdgcn_exp2f(s[st][i] - m_use);      // 2^(-inf) = 0 for masked keys
+                    lsum += s[st][i];
+                }
+            lsum = rows_sum(lsum);
+            const float alpha = (m_run[qg] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qg] - m_use);
+            l_run[qg] = l_run[qg] * alpha + lsum;
+            if (__any(m_new != m_run[qg])) {             // some row's maximum moved: rescale what is summed so far
+#pragma unroll
+                for (int dt = 0; dt < D16; ++dt) {
+                    acc[qg][dt][0] *= alpha;
+                    acc[qg][dt][1] *= alpha;
+                    acc[qg][dt][2] *= alpha;
+                    acc[qg][dt][3] *= alpha;
                 }
             }
+            m_run[qg] = m_new;
+#pragma unroll
+            for (int b = 0; b < BN / 32; ++b)
+                pw[qg][b] = uint4_t{pack2(s[2 * b][0], s[2 * b][1]), pack2(s[2 * b][2], s[2 * b][3]),
+                                    pack2(s[2 * b + 1][0], s[2 * b + 1][1]), pack2(s[2 * b + 1][2], s[2 * b + 1][3])};
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        // a row that sees no key yet (all of this pass lies above it or outside its window) keeps m = -inf
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        float lsum = 0.f;
-#pragma unroll
-        for (int st = 0; st < BN / 16; ++st)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                s[st][i] = __builtin_amdgcn_exp2f(s[st][i] - m_use);      // 2^(-inf) = 0 for masked keys
-                lsum += s[st][i];
-            }
-        lsum += __shfl_xor(lsum, 16, 64);
-        lsum += __shfl_xor(lsum, 32, 64);
-        const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_use);
-        l_run = l_run * alpha + lsum;
-        if (__any(m_new != m_run)) {                     // some row's maximum moved: rescale what is summed so far
-#pragma unroll
-            for (int dt = 0; dt < D16; ++dt) {
-                acc[dt][0] *= alpha;
-                acc[dt][1] *= alpha;
-                acc[dt][2] *= alpha;
-                acc[dt][3] *= alpha;
-            }
-        }
-        m_run = m_new;
 
-        // ---- O^T += V^T P^T, 32 keys per MFMA; V^T through the transposing LDS read
+        // ---- O^T += V^T P^T, 32 keys per MFMA; V^T through the transposing LDS read, once for every group
 #pragma unroll
         for (int b = 0; b < BN / 32; ++b) {
-            const uint4_t pw = {pack2(s[2 * b][0], s[2 * b][1]), pack2(s[2 * b][2], s[2 * b][3]),
-                                pack2(s[2 * b + 1][0], s[2 * b + 1][1]), pack2(s[2 * b + 1][2], s[2 * b + 1][3])};
-            const bf16x8_t pb = __builtin_bit_cast(bf16x8_t, pw);
             // this lane's address as lane l' = n of its group: key 32b + 4g + n/4, columns 4(n%4)..+3
             const uint16_t* vr = &v_cur[(32 * b + 4 * g + (n >> 2)) * VS + 4 * (n & 3)];
 #pragma unroll
@@ -276,8 +312,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + dt * 16));
                 const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(vr + 16 * VS + dt * 16));
                 const short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), pb, acc[dt], 0, 0, 0);
+#pragma unroll
+                for (int qg = 0; qg < QG; ++qg)
+                    acc[qg][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8_t, both), __builtin_bit_cast(bf16x8_t, pw[qg][b]), acc[qg][dt], 0, 0, 0);
             }
+        }
         }
         __syncthreads();                                 // every wave is done with this tile; the next one is complete
     }
@@ -285,16 +325,52 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #undef FETCH_ROW
 #undef STAGE_TO
 #undef ROW_OF
+#undef K_S
+#undef V_S
     MFMA_SETTLE();
-    // ---- acc[dt][i] = O^T[d = 16dt + 4g + i][query n]
-    if (q_ok) {
-        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-        bf16* op = out + ((size_t)(cu_q[seg] + q_local) * Hq + head) * D;
+    if constexpr (KSPLIT > 1) {
+        // the second group hands over what it has summed: per lane m, l and the accumulators, lane fastest
+        float* ms = reinterpret_cast<float*>(lds_raw) + (size_t)wave * QG * MERGE_SLOTS * 64 + lane;
+        if (grp == 1) {
+#pragma unroll
+            for (int qg = 0; qg < QG; ++qg) {
+                float* mq = ms + qg * MERGE_SLOTS * 64;
+                mq[0] = m_run[qg];
+                mq[64] = l_run[qg];
+#pragma unroll
+                for (int dt = 0; dt < D16; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) mq[(2 + 4 * dt + i) * 64] = acc[qg][dt][i];
+            }
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int qg = 0; qg < QG; ++qg) {
+            const float* mq = ms + qg * MERGE_SLOTS * 64;
+            const float m1 = mq[0], l1 = mq[64];
+            const float m = fmaxf(m_run[qg], m1);
+            const float a0 = (m_run[qg] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qg] - m);
+            const float a1 = (m1 == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+            l_run[qg] = l_run[qg] * a0 + l1 * a1;
+#pragma unroll
+            for (int dt = 0; dt < D16; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[qg][dt][i] = acc[qg][dt][i] * a0 + mq[(2 + 4 * dt + i) * 64] * a1;
+        }
+    }
+    // ---- acc[qg][dt][i] = O^T[d = 16dt + 4g + i][query n of group qg]
+#pragma unroll
+    for (int qg = 0; qg < QG; ++qg) {
+        if (!q_ok[qg]) continue;
+        const float inv = l_run[qg] > 0.f ? 1.0f / l_run[qg] : 0.f;
+        bf16* op = out + ((size_t)(cu_q[seg] + pos_q[qg] - pos0) * Hq + head) * D;
 #pragma unroll
         for (int dt = 0; dt < D16; ++dt) {
             uint2 w;
-            w.x = pack2(acc[dt][0] * inv, acc[dt][1] * inv);
-            w.y = pack2(acc[dt][2] * inv, acc[dt][3] * inv);
+            w.x = pack2(acc[qg][dt][0] * inv, acc[qg][dt][1] * inv);
+            w.y = pack2(acc[qg][dt][2] * inv, acc[qg][dt][3] * inv);
             *reinterpret_cast<uint2*>(op + dt * 16 + 4 * g) = w;
         }
     }
@@ -303,15 +379,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #define PRE_CAT2(a, b) a##b
 #define PRE_CAT(a, b) PRE_CAT2(a, b)
 // head sizes 16*(4*PRE_PART+1) .. 16*(4*PRE_PART+4)
-extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, dim3 grid, hipStream_t st, const bf16* q, bf16* out,
+extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out,
                                               const bf16* kp, const bf16* vp, const int* pt,
                                               const int* cup, const int* kvs, const int* cuq,
                                               const int* qs, const int* tiles, int n_tiles, int Hq,
                                               int Hkv, int P, float scale, int window) {
 #define PRE_CASE(N)                                                                               \
     case N:                                                                                       \
-        hipLaunchKernelGGL(attn_prefill_kernel<N>, grid, dim3(256), 0, st, q, out, kp, vp, pt, cup, \
-                           kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window);              \
+        if (key_split == 2 && N <= PRE_WIDE_D16)                                                      \
+            hipLaunchKernelGGL((attn_prefill_kernel<N, (N <= PRE_WIDE_D16 ? 2 : 1), (N <= PRE_WIDE_D16 ? 2 : 1)>), \
+                               grid, dim3(512), 0, st, q, out, kp, vp, pt, cup, kvs, cuq, qs, tiles,      \
+                               n_tiles, Hq, Hkv, P, scale, window);                                       \
+        else                                                                                          \
+            hipLaunchKernelGGL((attn_prefill_kernel<N, (N <= PRE_WIDE_D16 ? 2 : 1), 1>), grid, dim3(256), \
+                               0, st, q, out, kp, vp, pt, cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P,  \
+                               scale, window);                                                        \
         return RA_OK;
     switch (D16) {
         PRE_CASE(4 * PRE_PART + 1) PRE_CASE(4 * PRE_PART + 2) PRE_CASE(4 * PRE_PART + 3)
@@ -323,7 +405,7 @@ extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, dim3 grid, hipStream_t s
 #endif  // PRE_PART
 
 #ifdef PRE_API
-#define PRE_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
+#define PRE_PART_ARGS int D16, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
     const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs,    \
     const int* tiles, int n_tiles, int Hq, int Hkv, int P, float scale, int window
 extern "C" int ra_pre_part_0(PRE_PART_ARGS);
@@ -331,23 +413,33 @@ extern "C" int ra_pre_part_1(PRE_PART_ARGS);
 extern "C" int ra_pre_part_2(PRE_PART_ARGS);
 extern "C" int ra_pre_part_3(PRE_PART_ARGS);
 
+// Rows of a q tile for head size D: 128 up to head size 128, 64 beyond.
+extern "C" int ra_attention_prefill_tile_rows(int D) { return D <= 16 * PRE_WIDE_D16 ? 128 : 64; }
+
 // tiles: int32 [n_tiles][2] = (request number, first row of the tile within the request's new
-// tokens); every request with more than one new token is covered in tiles of 64 rows.
+// tokens); every request with more than one new token is covered in tiles of tile_rows rows,
+// which must be what ra_attention_prefill_tile_rows(D) says.
 extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k_pool,
                                          const void* v_pool, const int* page_table,
                                          const int* cu_pages, const int* kv_start, const int* cu_q,
-                                         const int* q_start, const int* tiles, int n_tiles, int Hq,
-                                         int Hkv, int D, int P, float scale, int window, void* stream) {
+                                         const int* q_start, const int* tiles, int n_tiles,
+                                         int tile_rows, int key_split, int Hq, int Hkv, int D, int P,
+                                         float scale, int window, void* stream) {
     if (n_tiles <= 0) return RA_OK;
     if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 ||
-        (long long)n_tiles * Hq > 0x7fffffffLL)
+        (long long)n_tiles * Hq > 0x7fffffffLL || tile_rows != ra_attention_prefill_tile_rows(D))
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(n_tiles * Hq);
     const int d16 = D / 16;
+    // key_split 2: a second group of waves takes every other key tile of each workgroup (head
+    // sizes up to 128; it pays when the workgroups are few and the longest tile decides the time).
+    // 0 decides here by the number of workgroups alone.
+    if (key_split <= 0) key_split = (long long)n_tiles * Hq <= 256 ? 2 : 1;
+    if (key_split > 2) return RA_ERR_ARG;
     int rc;
 #define GO(k)                                                                                      \
-    rc = ra_pre_part_##k(d16, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
+    rc = ra_pre_part_##k(d16, key_split, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tiles, \
                          n_tiles, Hq, Hkv, P, scale, window)
     switch ((d16 - 1) / 4) {

@@ -69,6 +69,26 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return t;
 }
 
+// Maximum and sum over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), the result
+// in every lane, by the lane swaps of gfx950: v_permlane16_swap exchanges the odd rows of its
+// first operand with the even rows of its second, v_permlane32_swap the upper half of the first
+// with the lower half of the second; with the same value in both operands the two results hold
+// the two partners of every lane. No LDS round trip as with a shuffle. The sum is
+// (row0 + row1) + (row2 + row3) in every lane.
+typedef unsigned ra_uint2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float rows_max(float v) {
+    ra_uint2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    ra_uint2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 static inline int ra_launch_status() {
     return hipGetLastError() == hipSuccess ? RA_OK : RA_ERR_LAUNCH;
 }

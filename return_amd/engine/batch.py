@@ -62,17 +62,18 @@ class StepBatch:
     n_prefill_tokens: int = 0
     prefill_toks: Optional[torch.Tensor] = None    # int32 token rows of the others; None: all rows
     prefill_segs: List[int] = dataclasses.field(default_factory=list)   # host: their request numbers
-    n_prefill_tiles: int = 0
-    prefill_tiles: Optional[torch.Tensor] = None   # int32 [tiles, 2]: request number, first row; 64 rows each
+    # q tiles of the prefill attention kernel, by rows per tile: rows -> int32 [tiles, 2] of
+    # (request number, first row of the tile among the request's new tokens)
+    prefill_tiles: dict = dataclasses.field(default_factory=dict)
 
 
-PREFILL_TILE_ROWS = 64      # query rows per workgroup of the prefill attention kernel
+PREFILL_TILE_ROWS = (64, 128)      # query rows per workgroup of the prefill attention kernel, by head size
 
 
-def prefill_tiles(q_lens, q_starts=None):
-    """(request number, first row) of every tile of PREFILL_TILE_ROWS rows, for requests with more
-    than one token; tiles that read the most keys come first, so the longest work starts earliest."""
-    tiles = [(i, off) for i, q in enumerate(q_lens) if q != 1 for off in range(0, q, PREFILL_TILE_ROWS)]
+def prefill_tiles(q_lens, q_starts=None, rows=64):
+    """(request number, first row) of every tile of ``rows`` rows, for requests with more than
+    one token; tiles that read the most keys come first, so the longest work starts earliest."""
+    tiles = [(i, off) for i, q in enumerate(q_lens) if q != 1 for off in range(0, q, rows)]
     if q_starts is not None:
         tiles.sort(key=lambda t: -(int(q_starts[t[0]]) + t[1]))
     return tiles
@@ -89,7 +90,8 @@ class StepBuilder:
         T, N, G = self.max_tokens, self.max_requests, len(cache.groups)
         layout = [("token_ids", T), ("positions", T), ("logit_rows", T), ("cu_q", N + 1),
                   ("q_start", N), ("seq_lens", N), ("slot_ids", N), ("decode_segs", N),
-                  ("prefill_toks", T), ("prefill_tiles", 2 * (T // PREFILL_TILE_ROWS + N))]
+                  ("prefill_toks", T)]
+        layout += [(f"prefill_tiles{rows}", 2 * (T // rows + N)) for rows in PREFILL_TILE_ROWS]
         for g in range(G):
             layout += [(f"slot_mapping{g}", T), (f"cu_pages{g}", N + 1), (f"kv_start{g}", N)]
         self._small_end = None
@@ -161,9 +163,11 @@ class StepBuilder:
             self._put(f"cu_pages{g}", gt.cu_pages)
             self._put(f"kv_start{g}", gt.kv_start)
             self._put(f"page_table{g}", gt.page_table)
-        tiles = prefill_tiles(tables.q_lens, tables.q_start)
-        if tiles:
-            self._put("prefill_tiles", np.asarray(tiles, dtype=np.int32).reshape(-1))
+        tiles = {}
+        if pre:
+            for rows in PREFILL_TILE_ROWS:
+                tiles[rows] = prefill_tiles(tables.q_lens, tables.q_start, rows)
+                self._put(f"prefill_tiles{rows}", np.asarray(tiles[rows], dtype=np.int32).reshape(-1))
         # one copy for the small tables, one per group for the used part of its page table
         self._dev[:self._small_end].copy_(self._host[:self._small_end], non_blocking=True)
         groups = []
@@ -196,5 +200,6 @@ class StepBuilder:
             max_decode_seq_len=max((int(tables.seq_lens[i]) for i in dec), default=0),
             n_prefill_tokens=n_pre_tok,
             prefill_toks=self._view("prefill_toks", n_pre_tok) if mixed_kinds else None,
-            prefill_segs=pre, n_prefill_tiles=len(tiles),
-            prefill_tiles=self._view("prefill_tiles", 2 * len(tiles)).view(-1, 2) if tiles else None)
+            prefill_segs=pre,
+            prefill_tiles={rows: self._view(f"prefill_tiles{rows}", 2 * len(t)).view(-1, 2)
+                           for rows, t in tiles.items()})

@@ -64,7 +64,8 @@ def _declare(lib):
         "ra_gemm_mfma_bf16": [P, P, P, I, I, I, I, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
-        "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P],
+        "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+        "ra_attention_prefill_tile_rows": [I],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
     }
     for name, args in sigs.items():
@@ -89,6 +90,7 @@ class HipOps:
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
         self.decode_split_tokens = 0         # keys per split of the decode attention; 0: by batch size
+        self.prefill_key_split = 0           # groups of waves that share a q tile's keys (1 or 2); 0: by the number of tiles
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
         self.own_gemm = False                # True: bf16 products of many rows use the hand-written MFMA kernel
@@ -341,16 +343,34 @@ class HipOps:
             toks, n_tok = step.prefill_toks, step.n_prefill_tokens
         else:
             toks, n_tok = None, T
-        if q.dtype == torch.bfloat16 and step.n_prefill_tiles > 0 and D % 16 == 0 and D <= 256 and \
+        if q.dtype == torch.bfloat16 and step.prefill_tiles and D % 16 == 0 and D <= 256 and \
                 (fast_decode or step.n_decode == 0):
+            rows = self.lib.ra_attention_prefill_tile_rows(D)
+            tiles = step.prefill_tiles.get(rows)
+            if tiles is None:
+                raise KernelError(f"attention: the step lists no q tiles of {rows} rows (head size {D})")
+            split = self.prefill_key_split or self._prefill_key_split(step, rows, tiles.shape[0] * n_q)
             self._check(self.lib.ra_attention_prefill_bf16(
-                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(step.prefill_tiles),
-                step.n_prefill_tiles, n_q, n_kv, D, P, float(scale), window, self._stream()),
+                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], rows,
+                split, n_q, n_kv, D, P, float(scale), window, self._stream()),
                 "attention_prefill_bf16")
             return
         self._check(self.lib.ra_attention_plain(
             _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
             n_q, n_kv, D, P, float(scale), window, _code(q.dtype), self._stream()), "attention_plain")
+
+    @staticmethod
+    def _prefill_key_split(step, rows, n_workgroups):
+        """Whether two groups of waves should share each q tile's keys (measured on MI355X): yes
+        while the workgroups do not fill the chip, and up to three per CU when the longest tile
+        reads far more keys than the average one, since then the longest tile decides the time."""
+        if n_workgroups <= 256:
+            return 2
+        if n_workgroups > 768:
+            return 1
+        ends = [s + min(off + rows, q) for q, s in zip(step.q_lens, step.q_starts) if q != 1
+                for off in range(0, q, rows)]
+        return 2 if max(ends) * len(ends) >= 1.4 * sum(ends) else 1
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, top_p, u):

@@ -245,9 +245,10 @@ def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
                  n_prefill_tokens=cu_q[-1] - len(dec),
                  prefill_toks=i32([t for i in pre for t in range(cu_q[i], cu_q[i + 1])]) if both else None,
                  prefill_segs=pre)
-    from return_amd.engine.batch import prefill_tiles
-    tiles = prefill_tiles(q_lens, q_starts)
-    extra.update(n_prefill_tiles=len(tiles), prefill_tiles=i32(tiles) if tiles else None)
+    from return_amd.engine.batch import PREFILL_TILE_ROWS, prefill_tiles
+    extra.update(prefill_tiles={})
+    if any(q != 1 for q in q_lens):
+        extra.update(prefill_tiles={rows: i32(prefill_tiles(q_lens, q_starts, rows)) for rows in PREFILL_TILE_ROWS})
     return types.SimpleNamespace(**extra, n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
                                  seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
                                  q_lens=list(q_lens), q_starts=list(q_starts),
@@ -297,13 +298,16 @@ def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
     torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("key_split", [1, 2])
 @pytest.mark.parametrize("D", list(range(16, 257, 16)))
-def test_prefill_attention_every_head_size(ops, ref, D):
+def test_prefill_attention_every_head_size(ops, ref, D, key_split, monkeypatch):
     """The bfloat16 prefill kernel at every head size it takes: whole prompts, portions with
-    context, tiles that end inside a page, a window."""
+    context, tiles that end inside a page, a window, an odd and an even number of key tiles;
+    with one group of waves per q tile and with two that share its keys."""
+    monkeypatch.setattr(ops, "prefill_key_split", key_split)
     for (Hq, Hkv), window in (((4, 2), 0), ((3, 1), 37)):
         P = 16
-        segs = [(70, 0), (2, 131), (65, 64), (5, 3)]
+        segs = [(70, 0), (2, 131), (65, 64), (5, 3), (130, 259), (140, 300)]
         need = [-(-(a + b) // P) for a, b in segs]
         pages_of, nxt = [], 0
         for k in need:
