@@ -59,6 +59,7 @@ class StepBatch:
     n_decode: int = 0
     decode_segs: Optional[torch.Tensor] = None     # int32 [n_decode] request numbers; None: all of them
     max_decode_seq_len: int = 0
+    decode_len_is_bound: bool = False              # max_decode_seq_len is an upper bound (a graph's bucket), not the longest length
     n_prefill_tokens: int = 0
     prefill_toks: Optional[torch.Tensor] = None    # int32 token rows of the others; None: all rows
     prefill_segs: List[int] = dataclasses.field(default_factory=list)   # host: their request numbers

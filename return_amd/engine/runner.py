@@ -182,14 +182,10 @@ class ModelRunner:
         key = (batch.n_seqs, bucket)
         entry = self._graphs.get(key)
         batch.max_decode_seq_len = bucket        # grid and scratch sizes cover the whole bucket
+        batch.decode_len_is_bound = True
         if entry is None:
-            ops = self.rt.ops
-            saved = getattr(ops, "decode_split_tokens", None)
-            if saved is not None and saved <= 0:
-                # the split size is part of the captured launch: fix it from the bucket
-                chunks = batch.n_seqs * max(1, self.model.max_kv_heads()) * (bucket // 64)
-                ops.decode_split_tokens = 64 * max(1, min(8, chunks // 4096))
-            split = getattr(ops, "decode_split_tokens", None)
+            # what a launch derives from the context length (grid, split size, scratch) now
+            # derives from the bucket, and so holds for every replay
             side = torch.cuda.Stream(self.rt.device)
             side.wait_stream(torch.cuda.current_stream(self.rt.device))
             with torch.cuda.stream(side):
@@ -201,11 +197,9 @@ class ModelRunner:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             with torch.cuda.graph(graph, pool=self._graph_pool):
                 logits, picked = self._decode_body(batch)
-            if saved is not None:
-                ops.decode_split_tokens = saved
-            entry = (graph, logits, picked, split)
+            entry = (graph, logits, picked)
             self._graphs[key] = entry
-        graph, logits, picked, _ = entry
+        graph, logits, picked = entry
         graph.replay()
         return logits, picked
 

@@ -325,9 +325,14 @@ class HipOps:
             longest = step.max_decode_seq_len
             S = self.decode_split_tokens
             if S <= 0:
-                # enough splits to fill the chip, few enough to keep the merge cheap
+                # about a thousand waves in all (four per CU) fill the chip; fewer, longer splits
+                # spend less on starting up and on the merge (measured from 1 to 128 requests)
                 chunks = step.n_decode * n_kv * ((longest + 63) // 64)
-                S = 64 * max(1, min(8, chunks // 4096))
+                S = 64 * max(2, -(-chunks // 1024))
+                if getattr(step, "decode_len_is_bound", False):
+                    # the lengths lie somewhere below `longest` (a graph's context bucket): splits
+                    # of at most an eighth of it keep the work of a request even
+                    S = min(S, max(128, longest // 8 // 64 * 64))
             max_splits = (longest - 1) // S + 1
             if window > 0:                       # a window spans at most this many splits
                 max_splits = min(max_splits, (window + S - 2) // S + 1)

@@ -60,11 +60,6 @@ class Decoder:
             raise ValueError(f"cache layers {sorted(missing)} are read but never written")
         return need
 
-    def max_kv_heads(self):
-        """Most kv heads of any paged cache layer (sizing hint for the decode attention's splits)."""
-        heads = [spec.num_kv_heads for spec in self.cache_layers().values() if hasattr(spec, "num_kv_heads")]
-        return max(heads) if heads else 1
-
     def forward(self, step, cache):
         """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
         h = self.embedding.forward(step.token_ids)
