@@ -62,6 +62,8 @@ def _declare(lib):
         "ra_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, P],
         "ra_gemm_skinny_gated_bf16": [P, P, P, I, I, I, P],
         "ra_gemm_mfma_bf16": [P, P, P, I, I, I, I, P],
+        "ra_gemm_resident_bf16": [P, P, P, I, I, I, I, I, I, P],
+        "ra_gemm_resident_fits": [I, I, I],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
@@ -103,6 +105,17 @@ class HipOps:
         if out_dtype == torch.float32:
             return M <= 16                   # more rows: the tiled MFMA product (the library has no bf16-in, fp32-out product)
         return M <= 4 or (M <= 16 and N * K <= (32 << 20))
+
+    def use_resident(self, M, N, K, gated):
+        """Whether the product with x resident in LDS beats the skinny product for x [M, K] and
+        N result columns (measured on MI355X): from two rows on, when every workgroup gets
+        several tiles of 16 columns; one row and few tiles are the skinny product's."""
+        if not self.lib.ra_gemm_resident_fits(M, K, 1 if gated else 0):
+            return False
+        tiles = -(-N // 16)
+        if 2 <= M <= 8:
+            return tiles >= 384
+        return M > 8 and tiles >= 2048
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -269,6 +282,12 @@ class HipOps:
         if w.shape[1] != K:
             raise KernelError(f"linear: x {tuple(x.shape)} times weight {tuple(w.shape)}^T")
         out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.bfloat16 and out_dtype in (torch.bfloat16, torch.float32) and \
+                self.use_resident(M, N, K, False):
+            y = torch.empty(M, N, dtype=out_dtype, device=self.device)
+            self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, _code(out_dtype),
+                                                       512 if M <= 8 else 256, self._stream()), "gemm_resident")
+            return y
         if x.dtype == torch.bfloat16 and M > 0 and self.use_skinny(M, N, K, out_dtype):
             y = torch.empty(M, N, dtype=out_dtype, device=self.device)
             self._check(self.lib.ra_gemm_skinny_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
@@ -295,6 +314,11 @@ class HipOps:
         if w_gate_up.shape[1] != K or w_gate_up.shape[0] != 2 * I:
             raise KernelError(f"linear_silu_mul: x {tuple(x.shape)}, weight {tuple(w_gate_up.shape)}")
         out = torch.empty(M, I, dtype=x.dtype, device=self.device)
+        if x.dtype == torch.bfloat16 and self.use_resident(M, I, K, True):
+            self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K, 1,
+                                                       _code(x.dtype), 512 if M <= 8 else 256, self._stream()),
+                        "gemm_resident_gated")
+            return out
         if x.dtype == torch.bfloat16 and 0 < M <= self.gated_skinny_rows and K % 8 == 0:
             self._check(self.lib.ra_gemm_skinny_gated_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K,
                                                            self._stream()), "gemm_skinny_gated")

@@ -194,6 +194,32 @@ def test_skinny_product_fp32_out(ops, M, N, K):
     torch.testing.assert_close(y.double(), x.double() @ w.double().t(), atol=1e-4 * K ** 0.5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("M", [1, 2, 7, 8, 9, 16])
+@pytest.mark.parametrize("N,K,grid", [(331, 120, 0), (1000, 264, 7), (48, 4096, 0), (6200, 72, 512)])
+def test_resident_product(ops, ref, M, N, K, grid):
+    """The product with x resident in LDS, called directly: bf16 and fp32 results, the gated
+    form, more tiles than workgroups, widths that are no multiple of the tile."""
+    from return_amd.kernels.hip_ops import _code, _ptr
+    st = torch.cuda.current_stream().cuda_stream
+    x = rnd(M, K, dtype=torch.bfloat16, seed=3)
+    w = rnd(2 * N, K, dtype=torch.bfloat16, seed=4) * 0.2
+    want = x.double() @ w.double().t()
+    for out_dtype in (torch.bfloat16, torch.float32):
+        y = torch.full((M, N), 7.0, dtype=out_dtype, device=DEV)
+        assert ops.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, _code(out_dtype), grid, st) == 0
+        if out_dtype == torch.float32:
+            torch.testing.assert_close(y.double(), want[:, :N], atol=1e-4 * K ** 0.5, rtol=1e-5)
+        else:
+            torch.testing.assert_close(y.float(), want[:, :N].float(), **tol(torch.bfloat16))
+    y = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    assert ops.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 1, _code(torch.bfloat16), grid, st) == 0
+    g, u = want[:, :N], want[:, N:]
+    torch.testing.assert_close(y.float(), (g * torch.sigmoid(g) * u).float(), **tol(torch.bfloat16))
+    # what does not fit is refused, not computed
+    assert ops.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), 17, N, K, 0, _code(torch.bfloat16), grid, st) != 0
+    assert not ops.lib.ra_gemm_resident_fits(16, 8192, 0) and ops.lib.ra_gemm_resident_fits(8, 8192, 0)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(65, 331, 120), (128, 128, 32), (129, 257, 264), (300, 1000, 512), (70, 48, 8)])
 def test_tiled_mfma_product(ops, out_dtype, M, N, K):
