@@ -99,12 +99,13 @@ class HipOps:
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
-        (measured on MI355X: it wins for one to four rows, and up to 16 rows on small weights)."""
+        (measured on MI355X: it wins for one to four rows, up to 16 rows on small weights and up
+        to 32 rows on the smallest)."""
         if K % 8 or M > 64:
             return False
         if out_dtype == torch.float32:
             return M <= 16                   # more rows: the tiled MFMA product (the library has no bf16-in, fp32-out product)
-        return M <= 4 or (M <= 16 and N * K <= (32 << 20))
+        return M <= 4 or (M <= 16 and N * K <= (32 << 20)) or (M <= 32 and N * K <= (16 << 20))
 
     def use_resident(self, M, N, K, gated):
         """Whether the product with x resident in LDS beats the skinny product for x [M, K] and
