@@ -96,6 +96,11 @@ class HipOps:
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
         self.own_gemm = False                # True: bf16 products of many rows use the hand-written MFMA kernel
+        try:                                 # whether the library multiplies bf16 operands into fp32 results
+            a = torch.ones(1, 8, dtype=torch.bfloat16, device=self.device)
+            self._library_fp32_out = torch.mm(a, a.t(), out_dtype=torch.float32).dtype == torch.float32
+        except (TypeError, RuntimeError):
+            self._library_fp32_out = False
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -104,7 +109,7 @@ class HipOps:
         if K % 8 or M > 64:
             return False
         if out_dtype == torch.float32:
-            return M <= 16                   # more rows: the tiled MFMA product (the library has no bf16-in, fp32-out product)
+            return M <= 16                   # more rows: the library, or the tiled MFMA product
         return M <= 4 or (M <= 16 and N * K <= (32 << 20)) or (M <= 32 and N * K <= (16 << 20))
 
     def use_resident(self, M, N, K, gated):
@@ -296,6 +301,9 @@ class HipOps:
             return y
         if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and M > 0 and not self.own_gemm:
             return torch.matmul(x, w.t())          # library product, as the reference's F.linear
+        if x.dtype == torch.bfloat16 and out_dtype == torch.float32 and M > 0 and not self.own_gemm \
+                and self._library_fp32_out:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)   # bf16 operands, 32-bit sums and results
         if x.dtype == torch.bfloat16 and M > 0 and K % 8 == 0:
             y = torch.empty(M, N, dtype=out_dtype, device=self.device)
             self._check(self.lib.ra_gemm_mfma_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),

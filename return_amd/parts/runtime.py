@@ -38,9 +38,10 @@ class Runtime:
         key = (t.data_ptr(), tuple(t.shape), t.dtype)
         hit = self._cast.get(key)
         if hit is None:
-            hit = t.to(device=self.device, dtype=self.dtype).contiguous()
+            # the stored tensor is kept too: while it lives, its address cannot go to another tensor
+            hit = (t, t.to(device=self.device, dtype=self.dtype).contiguous())
             self._cast[key] = hit
-        return hit
+        return hit[1]
 
     def vector32(self, t: torch.Tensor) -> torch.Tensor:
         """A small vector (norm weight) as 32-bit floats; bf16 values convert exactly."""

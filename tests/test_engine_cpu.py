@@ -91,3 +91,21 @@ def test_step_checks(folder_a):
     assert runner.cache.seq_len("a") == 3
     with pytest.raises(ValueError, match="max_position"):
         runner.step([StepEntry("a", [1] * 300, [])])
+
+
+def test_prepared_matrices_follow_the_tensor_not_its_address():
+    """Runtime.matrix keeps one prepared copy per stored tensor (tied weights stay one copy); a
+    tensor that is freed and another of the same shape at the same address must not get it."""
+    from return_amd.parts.runtime import Runtime
+    from tests.torch_ops import TorchOps
+    rt = Runtime("cpu", "bfloat16", ops=TorchOps("cpu"))     # float32 stored, bfloat16 prepared: a copy
+    t = torch.full((64, 80), 1.0)
+    assert rt.matrix(t) is rt.matrix(t) and rt.matrix(t).dtype == torch.bfloat16
+    seen = set()
+    for i in range(200):
+        t = torch.full((64, 80), float(i))
+        seen.add(t.data_ptr())
+        assert float(rt.matrix(t)[3, 5]) == float(i)
+        del t
+    rt.forget_casts()
+    assert not rt._cast
