@@ -7,7 +7,7 @@
 // walks over tiles of 16 rows of W (tile = blockIdx.x, += gridDim.x): its waves split K in
 // blocks of 256, W is the A operand of MFMA 16x16x32 bf16 read straight from memory (lane
 // (n, g): 16 bytes of row n at k0 + 8g), x the B operand read from LDS, and the waves' partial
-// tiles are added through LDS in wave order. x is read from the cache once per workgroup
+// tiles are added through LDS in wave order (one barrier, then every thread adds one element). x is read from the cache once per workgroup
 // instead of once per tile, and the loop issues no loads but W's.
 // Results: bfloat16 or fp32 [M, N]; GATED (W = [Wg; Wu], rollout/monkey_patch/qwen3.py:103):
 // silu(g) * u as [M, N] (rollout/fused.py:103-114).
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_resident_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int XS = K + 8;                                       // row stride of x in LDS (elements)
     uint16_t* x_s = reinterpret_cast<uint16_t*>(lds_raw);
-    float* red = reinterpret_cast<float*>(lds_raw + (size_t)MP * XS * 2);   // [NG][MB][16][17]
+    float* red = reinterpret_cast<float*>(lds_raw + (size_t)MP * XS * 2);   // [WAVES][NG][16][MP + 1]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
@@ -81,32 +81,29 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_resident_kernel(
             }
         }
         MFMA_SETTLE();
-        // c[z][b][i] = partial y[m = 16b + n][row n0 + 4g + i]; the waves add theirs in order
+        // c[z][0][i] = partial y[m = n][row n0 + 4g + i]: every wave puts its tile down, then the
+        // threads add the waves' tiles in wave order
+        if (n < MP) {
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) {
-            if (wave == w) {
+            for (int z = 0; z < NG; ++z)
 #pragma unroll
-                for (int z = 0; z < NG; ++z)
-#pragma unroll
-                    for (int b = 0; b < MB; ++b)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            float* p = &red[((z * MB + b) * 16 + 4 * g + i) * 17 + n];
-                            *p = (w == 0) ? c[z][b][i] : *p + c[z][b][i];
-                        }
-            }
-            __syncthreads();
+                for (int i = 0; i < 4; ++i) red[((wave * NG + z) * 16 + 4 * g + i) * (MP + 1) + n] = c[z][0][i];
         }
-        for (int e = tid; e < MB * 256; e += WAVES * 64) {
-            const int b = e >> 8, mm = (e >> 4) & 15, r = e & 15;     // r fastest: neighbours write neighbours
-            const int m = b * 16 + mm, col = n0 + r;
-            if (m < M && col < N) {
-                float s = red[((0 * MB + b) * 16 + r) * 17 + mm];
+        __syncthreads();
+        for (int e = tid; e < MP * 16; e += WAVES * 64) {
+            const int mm = e >> 4, r = e & 15;                // r fastest: neighbours write neighbours
+            const int col = n0 + r;
+            if (mm < M && col < N) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) s += red[((w * NG + 0) * 16 + r) * (MP + 1) + mm];
                 if constexpr (GATED) {
-                    const float up = red[((1 * MB + b) * 16 + r) * 17 + mm];
+                    float up = 0.f;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) up += red[((w * NG + 1) * 16 + r) * (MP + 1) + mm];
                     s = s / (1.0f + expf(-s)) * up;           // gate and up stay 32-bit until here
                 }
-                out[(size_t)m * N + col] = from_f<TO>(s);
+                out[(size_t)mm * N + col] = from_f<TO>(s);
             }
         }
         __syncthreads();
@@ -131,7 +128,7 @@ static int launch_resident(int grid, size_t lds, hipStream_t st, const bf16* x, 
 // LDS bytes for x [M, K] (M rounded up to 8 or 16) plus the reduction buffer
 static size_t resident_lds(int M, int K, bool gated) {
     const int mp = M <= 8 ? 8 : 16;
-    return (size_t)mp * (K + 8) * 2 + (size_t)(gated ? 2 : 1) * 16 * 17 * 4;
+    return (size_t)mp * (K + 8) * 2 + (size_t)8 * (gated ? 2 : 1) * 16 * (mp + 1) * 4;
 }
 
 extern "C" int ra_gemm_resident_fits(int M, int K, int gated) {
