@@ -371,6 +371,46 @@ def test_decode_attention_every_head_size(ops, ref, D):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_len", [1, 2, 7, 70])
+@pytest.mark.parametrize("older_wins", [True, False])
+def test_attention_edges_of_window_and_causality(ops, dtype, q_len, older_wins):
+    """Keys are made so that one edge of what a query may see decides its output. older_wins: the
+    score grows with the key's age, so every query row picks the oldest key of its window and a
+    window that is one key too long or too short shows; else it grows with the position, every row
+    picks itself, and a row that sees the key after it shows. The edges of the rows straddle page
+    borders, the pages lie scattered; one token goes to the decode kernel, more to the prefill kernel."""
+    Hq, Hkv, D, P, window = 4, 2, 64, 16, 37
+    start = 220 - q_len                                  # the last row sits at position 219
+    L = start + q_len
+    n_pages = -(-L // P)
+    perm = torch.randperm(n_pages + 5, generator=torch.Generator().manual_seed(9)).tolist()
+    pages = perm[:n_pages]
+    step = _step([q_len], [start], P, [pages])
+    pos = torch.arange(L)
+    mag = (256 - pos if older_wins else pos + 1).float()         # whole numbers up to 256: exact in bfloat16
+    k = torch.zeros(L, Hkv, D)
+    k[:, :, 0] = mag[:, None]
+    v = rnd(L, Hkv, D, seed=71).cpu()
+    kp = torch.zeros(n_pages + 5, P, Hkv, D)
+    vp = torch.zeros_like(kp)
+    for i in range(L):
+        kp[pages[i // P], i % P] = k[i]
+        vp[pages[i // P], i % P] = v[i]
+    kp, vp = kp.to(dtype).to(DEV), vp.to(dtype).to(DEV)
+    q = torch.zeros(q_len, Hq, D)
+    q[:, :, 0] = 96.0                                    # 96 * 1 / sqrt(64) = 12 per step of the magnitude
+    q = q.to(dtype).to(DEV)
+    out = torch.zeros_like(q)
+    ops.attention(q, out, kp, vp, step, 0, D ** -0.5, window)
+    for r in range(q_len):
+        pos_q = start + r
+        pick = max(0, pos_q - window + 1) if older_wins else pos_q
+        want = v[pick].to(dtype).float().repeat_interleave(Hq // Hkv, dim=0)      # [Hq, D]
+        torch.testing.assert_close(out[r].float().cpu(), want, atol=2e-2 if dtype == torch.bfloat16 else 1e-4,
+                                   rtol=0, msg=lambda m: f"row {r} (position {pos_q}) should have picked key {pick}: {m}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_far_key_stands_out(ops, dtype):
     """One key far back among hundreds is made to dominate: the output must be its value."""
     Hq, Hkv, D, P, L = 4, 2, 64, 16, 700
