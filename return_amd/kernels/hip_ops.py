@@ -361,7 +361,7 @@ class HipOps:
                 # about two thousand waves in all (eight per CU) fill the chip; fewer, longer
                 # splits spend less on starting up and on the merge (measured from 1 to 128 requests)
                 chunks = step.n_decode * n_kv * ((longest + 63) // 64)
-                S = 64 * max(2, -(-chunks // 2048))
+                S = 64 * max(2, -(-chunks // 2048), -(-longest // 4096))     # and at most 64 splits a request
                 if getattr(step, "decode_len_is_bound", False):
                     # the lengths lie somewhere below `longest` (a graph's context bucket): splits
                     # of at most an eighth of it keep the work of a request even
