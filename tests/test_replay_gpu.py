@@ -98,3 +98,37 @@ def test_long_decoding(folder_b):
     steps = tt.tail_decoded(reqs, tail=300)
     runner = make_runner(folder_b, "float32", 320)
     compare(tt.run_in_process(runner, steps), want, reqs, "float32")
+
+
+ODD = [
+    # head size, heads, kv heads, width, intermediate, vocabulary, layers, page, tied
+    (240, 6, 3, 100, 100, 331, 2, 4, True),       # width no multiple of 8: the plain product; a page of 4
+    (16, 60, 3, 96, 328, 1000, 2, 8, True),       # 20 query heads to a kv head: beyond the decode kernel's 16
+    (80, 7, 1, 100, 48, 1000, 1, 32, False),      # 7 heads on one kv head, head size 80
+    (256, 5, 5, 136, 100, 97, 2, 48, False),      # the largest head size, a page of 48
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("D,Hq,Hkv,H,I,V,L,page,tied", ODD)
+def test_odd_configurations(tmp_path, dtype, D, Hq, Hkv, H, I, V, L, page, tied):
+    """Sizes at the edges of what the kernels take, or beyond (then the plain kernels must step in):
+    a mixed trace with page reuse against the plain implementation."""
+    import return_amd.models  # noqa: F401
+    from return_amd.config import lookup_architecture
+    from return_amd.weights import write_model_folder
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=V, hidden_size=H,
+               num_hidden_layers=L, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D,
+               intermediate_size=I, max_position_embeddings=256, rms_norm_eps=3e-4, rope_theta=5e4,
+               tie_word_embeddings=tied)
+    cls, _ = lookup_architecture("Qwen3ForCausalLM")
+    folder = str(tmp_path / "model")
+    write_model_folder(folder, cls.from_dict(raw), dtype="bfloat16", seed=D, std=0.05, embedding_std=0.05,
+                       norm_jitter=0.03)
+    reqs = {rid: tt.random_tokens(V, n, seed=ord(rid)) for rid, n in
+            {"a": 5, "b": 70, "c": 33, "d": 130, "e": 64, "f": 2, "g": 1}.items()}
+    want = oracle(folder, reqs)
+    steps = tt.mixed(reqs, seed=D)
+    runner = make_runner(folder, dtype, tt.peak_tokens(steps, page) + 2 * page, page)
+    compare(tt.run_in_process(runner, steps), want, reqs, dtype)
+    assert not runner.cache.live
