@@ -94,23 +94,37 @@ def seat_requests(runner, batch, context, seed=1):
 
 
 def decode_steps(runner, ids, steps, warmup, vocab):
-    """warmup untimed steps, then exactly ``steps`` timed; returns seconds."""
+    """warmup untimed steps, then exactly ``steps`` timed; returns seconds. As the engine decodes:
+    every step is launched before the one before it is collected, its tokens taken over on the device."""
     import torch
-    from return_amd.engine import StepEntry
     n = len(ids)
     toks = [(7 * i + 3) % vocab for i in range(n)]
-    zeros, ones = [0.0] * n, [1.0] * n
+    zeros, ones, rows = [0.0] * n, [1.0] * n, list(range(n))
 
-    def one():
-        nonlocal toks
-        toks, _, _ = runner.decode_and_sample(ids, toks, zeros, [0] * n, ones, zeros)
+    launched = 0
 
-    for _ in range(warmup):
-        one()
+    def launch():
+        nonlocal launched
+        first = launched == 0
+        launched += 1
+        return runner.decode_launch(ids, toks if first else None, zeros, [0] * n, ones, zeros,
+                                    feed_rows=None if first else rows)
+
+    def run(count):
+        """count steps, each launched before the one before it is collected; all collected at the end"""
+        ticket = None
+        for _ in range(count):
+            ahead = launch()
+            if ticket is not None:
+                runner.decode_collect(ticket)
+            ticket = ahead
+        if ticket is not None:
+            runner.decode_collect(ticket)
+
+    run(warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        one()
+    run(steps)
     torch.cuda.synchronize()
     return time.perf_counter() - t0
 

@@ -76,13 +76,25 @@ class PagedGroup:
 
 
 class _Live:
-    __slots__ = ("slot", "seq_len", "pages", "first_pos")
+    __slots__ = ("slot", "seq_len", "pages", "first_pos", "_pages_np")
 
     def __init__(self, slot: int, n_groups: int):
         self.slot = slot
         self.seq_len = 0
         self.pages: List[List[int]] = [[] for _ in range(n_groups)]
         self.first_pos: List[int] = [0] * n_groups
+        self._pages_np: List[Optional[np.ndarray]] = [None] * n_groups
+
+    def pages_array(self, g: int) -> np.ndarray:
+        """pages[g] as an int32 array, made again only after pages_changed(g)."""
+        a = self._pages_np[g]
+        if a is None:
+            a = np.asarray(self.pages[g], dtype=np.int32)
+            self._pages_np[g] = a
+        return a
+
+    def pages_changed(self, g: int) -> None:
+        self._pages_np[g] = None
 
 
 class CacheManager:
@@ -230,14 +242,19 @@ class CacheManager:
                     f"of {grp.num_pages} are free")
 
         q_lens = [int(n_new) for _, n_new in entries]
+        lives = [self.live[rid] for rid, _ in entries]
         total = sum(q_lens)
         cu_q = np.zeros(n + 1, dtype=np.int32)
         cu_q[1:] = np.cumsum(q_lens)
-        q_start = np.array([self.live[rid].seq_len for rid, _ in entries], dtype=np.int32)
-        positions = np.empty(total, dtype=np.int32)
-        for i in range(n):
-            positions[cu_q[i]:cu_q[i + 1]] = np.arange(q_start[i], q_start[i] + q_lens[i])
-        slot_ids = np.array([self.live[rid].slot for rid, _ in entries], dtype=np.int32)
+        q_start = np.array([r.seq_len for r in lives], dtype=np.int32)
+        single = total == n                                   # one token each: a decode step
+        if single:
+            positions = q_start.copy()
+        else:
+            positions = np.empty(total, dtype=np.int32)
+            for i in range(n):
+                positions[cu_q[i]:cu_q[i + 1]] = np.arange(q_start[i], q_start[i] + q_lens[i])
+        slot_ids = np.array([r.slot for r in lives], dtype=np.int32)
 
         groups = []
         for g, grp in enumerate(self.groups):
@@ -245,21 +262,24 @@ class CacheManager:
             cu_pages = np.zeros(n + 1, dtype=np.int32)
             kv_start = np.zeros(n, dtype=np.int32)
             tables = []
-            for i, (rid, n_new) in enumerate(entries):
-                r = self.live[rid]
-                need = self._need(r, g, n_new)
+            for i, r in enumerate(lives):
+                need = self._need(r, g, q_lens[i])
                 if need:
                     r.pages[g].extend(grp.pages.take_many(need))
+                    r.pages_changed(g)
                     self.version += 1
-                pages = np.asarray(r.pages[g], dtype=np.int32)
-                pos = positions[cu_q[i]:cu_q[i + 1]]
-                rel = pos - r.first_pos[g]
-                slot_mapping[cu_q[i]:cu_q[i + 1]] = pages[rel // P] * P + rel % P
+                pages = r.pages_array(g)
+                if single:
+                    rel = r.seq_len - r.first_pos[g]
+                    slot_mapping[i] = r.pages[g][rel // P] * P + rel % P
+                else:
+                    rel = positions[cu_q[i]:cu_q[i + 1]] - r.first_pos[g]
+                    slot_mapping[cu_q[i]:cu_q[i + 1]] = pages[rel // P] * P + rel % P
                 tables.append(pages)
                 cu_pages[i + 1] = cu_pages[i] + len(pages)
                 kv_start[i] = r.first_pos[g]
             page_table = np.concatenate(tables) if tables else np.zeros(0, dtype=np.int32)
-            groups.append(GroupTables(slot_mapping, page_table.astype(np.int32), cu_pages, kv_start))
+            groups.append(GroupTables(slot_mapping, page_table, cu_pages, kv_start))
 
         for rid, n_new in entries:
             self.live[rid].seq_len += n_new
@@ -312,6 +332,7 @@ class CacheManager:
                 if drop:
                     grp.pages.give_back(r.pages[g][:drop])
                     del r.pages[g][:drop]
+                    r.pages_changed(g)
                     r.first_pos[g] += drop * P
                     self.version += 1
         self._step_requests = []
@@ -339,6 +360,7 @@ class CacheManager:
             assert not set(free) & set(held), f"group {g}: a page is both free and held"
             assert set(free) | set(held) == set(range(grp.num_pages)), f"group {g}: a page is lost"
             for rid, r in self.live.items():
+                assert r._pages_np[g] is None or r._pages_np[g].tolist() == r.pages[g], f"{rid!r}: stale page array"
                 assert r.first_pos[g] % P == 0
                 end = r.first_pos[g] + len(r.pages[g]) * P
                 assert r.seq_len <= end, f"{rid!r}: {r.seq_len} tokens but pages end at {end}"

@@ -53,6 +53,7 @@ class Engine:
         self.scheduler = Scheduler(runner.cache, ec.max_reside, ec.max_step_tokens, ec.prefill_chunk,
                                    runner.max_position)
         self._submitted = 0
+        self._in_flight = None              # (ticket, plan) of a decode step that was launched and not yet collected
         # running totals as in rollout/engine.py:84-125
         self.prefill_tokens = 0
         self.decode_tokens = 0
@@ -74,43 +75,75 @@ class Engine:
         return r
 
     # ------------------------------------------------------------------ one step
+    def _launch_decode(self, plan, previous=None):
+        """Start a decode-only plan. previous: the plan whose sampled tokens, still on the device,
+        are this plan's tokens (its rows are looked up by request)."""
+        rows = [e.request for e in plan.entries]
+        if previous is None:
+            tokens, feed = [e.tokens[0] for e in plan.entries], None
+        else:
+            row_of = {e.request.id: i for i, e in enumerate(previous.entries)}
+            tokens, feed = None, [row_of[r.id] for r in rows]
+        return self.runner.decode_launch(
+            [r.id for r in rows], tokens, [r.params.temperature for r in rows],
+            [r.params.top_k for r in rows], [r.params.top_p for r in rows],
+            [r.stream.next() for r in rows], feed_rows=feed)
+
+    def _book(self, plan, sampled, t0):
+        for e in plan.entries:
+            if e.request.finished:
+                continue
+            if len(e.tokens) == 1 and e.request.output:
+                self.decode_tokens += 1
+            else:
+                self.prefill_tokens += len(e.tokens)
+        ended = self.scheduler.finish_step(plan, sampled)
+        self.step_seconds += time.perf_counter() - t0
+        self.steps += 1
+        return ended
+
     def step(self) -> List[Request]:
-        """One scheduler step; returns the requests that ended in it (finished or failed)."""
+        """One scheduler step; returns the requests that ended in it (finished or failed).
+
+        A decode-only step is launched and collected in two halves: while it runs, the step
+        after it is decided and launched if it can be decided without the tokens
+        (Scheduler.schedule_ahead), so that the device does not wait for the host between steps.
+        """
+        t0 = time.perf_counter()
+        if self._in_flight is not None:
+            ticket, plan = self._in_flight
+            ahead = self.scheduler.schedule_ahead(plan) if self.config.lookahead else None
+            next_ticket = self._launch_decode(ahead, previous=plan) if ahead is not None else None
+            toks, logps = self.runner.decode_collect(ticket)
+            sampled = {e.request.id: (t, lp) for e, t, lp in zip(plan.entries, toks, logps)}
+            ended = self._book(plan, sampled, t0)
+            self._in_flight = (next_ticket, ahead) if ahead is not None else None
+            return ended
         plan = self.scheduler.schedule()
         ended = list(plan.failed)
         if not plan.entries:
             return ended
-        t0 = time.perf_counter()
-        sampled: Dict[object, tuple] = {}
-        rows = [e.request for e in plan.entries if e.sample]
-        if len(rows) == len(plan.entries) and all(len(e.tokens) == 1 for e in plan.entries):
+        if all(e.sample and len(e.tokens) == 1 for e in plan.entries):
             # decode only: one call that runs the model and the sampler (from a graph if enabled)
-            toks, logps, _ = self.runner.decode_and_sample(
-                [r.id for r in rows], [e.tokens[0] for e in plan.entries],
-                [r.params.temperature for r in rows], [r.params.top_k for r in rows],
-                [r.params.top_p for r in rows], [r.stream.next() for r in rows])
-            for r, t, lp in zip(rows, toks, logps):
-                sampled[r.id] = (t, lp)
-            rows = []
-        else:
-            entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
-                       for e in plan.entries]
-            logits = self.runner.step(entries)
+            ticket = self._launch_decode(plan)
+            if self.config.lookahead:
+                self._in_flight = (ticket, plan)
+                return ended + self.step()
+            toks, logps = self.runner.decode_collect(ticket)
+            sampled = {e.request.id: (t, lp) for e, t, lp in zip(plan.entries, toks, logps)}
+            return ended + self._book(plan, sampled, t0)
+        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
+                   for e in plan.entries]
+        logits = self.runner.step(entries)
+        rows = [e.request for e in plan.entries if e.sample]
+        sampled: Dict[object, tuple] = {}
         if rows:
             toks, logps = self.runner.sample(
                 logits, [r.params.temperature for r in rows], [r.params.top_k for r in rows],
                 [r.params.top_p for r in rows], [r.stream.next() for r in rows])
             for r, t, lp in zip(rows, toks, logps):
                 sampled[r.id] = (t, lp)
-        for e in plan.entries:
-            if len(e.tokens) == 1 and e.request.output:
-                self.decode_tokens += 1
-            else:
-                self.prefill_tokens += len(e.tokens)
-        ended += self.scheduler.finish_step(plan, sampled)
-        self.step_seconds += time.perf_counter() - t0
-        self.steps += 1
-        return ended
+        return ended + self._book(plan, sampled, t0)
 
     # ------------------------------------------------------------------ whole jobs
     def generate(self, prompts: Sequence[Sequence[int]],
@@ -122,7 +155,7 @@ class Engine:
         if len(params) != len(prompts):
             raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling parameter sets")
         requests = [self.submit(p, sp) for p, sp in zip(prompts, params)]
-        while self.scheduler.has_work():
+        while self.scheduler.has_work() or self._in_flight is not None:
             before = (self.steps, len(self.scheduler.waiting), len(self.scheduler.running))
             self.step()
             if before == (self.steps, len(self.scheduler.waiting), len(self.scheduler.running)):

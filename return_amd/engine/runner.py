@@ -71,6 +71,16 @@ class ModelRunner:
         self._samp_host_k = torch.zeros(n, dtype=torch.int32, pin_memory=pin)
         self._samp_dev_f = torch.zeros(3, n, dtype=torch.float32, device=self.rt.device)
         self._samp_dev_k = torch.zeros(n, dtype=torch.int32, device=self.rt.device)
+        self._samp_copied = torch.cuda.Event() if pin else None      # the staging above has left for the device
+        # Launch and collection of a decode step are two calls, so that the next step can be
+        # launched before this one's tokens are read: two pinned result buffers, the tokens of
+        # the last launch kept on the device for the next one to pick up.
+        self._picked_host = [torch.zeros(n, 2, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self._picked_ready = [torch.cuda.Event() if pin else None for _ in range(2)]
+        self._feed_host = torch.zeros(n, dtype=torch.int64, pin_memory=pin)
+        self._feed_dev = torch.zeros(n, dtype=torch.int64, device=self.rt.device)
+        self._launches = 0
+        self._last_picked: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request_id) -> None:
@@ -120,12 +130,16 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ decode from a graph
     def _put_sampling(self, m, temperature, top_k, top_p, uniforms):
+        if self._samp_copied is not None:
+            self._samp_copied.synchronize()          # the last launch's options have left the staging buffer
         self._samp_host_f[0, :m] = torch.as_tensor(temperature, dtype=torch.float32)
         self._samp_host_f[1, :m] = torch.as_tensor(top_p, dtype=torch.float32)
         self._samp_host_f[2, :m] = torch.as_tensor(uniforms, dtype=torch.float32)
         self._samp_host_k[:m] = torch.as_tensor(top_k, dtype=torch.int32)
         self._samp_dev_f.copy_(self._samp_host_f, non_blocking=True)
         self._samp_dev_k.copy_(self._samp_host_k, non_blocking=True)
+        if self._samp_copied is not None:
+            self._samp_copied.record()
 
     def _decode_body(self, batch):
         logits = self.model.forward(batch, self.cache)
@@ -134,17 +148,27 @@ class ModelRunner:
                                     self._samp_dev_f[1, :m], self._samp_dev_f[2, :m])
         return logits, picked
 
-    def decode_and_sample(self, request_ids, tokens, temperature, top_k, top_p, uniforms):
-        """One token per request, logits sampled at once: the steady state of generation.
+    def decode_launch(self, request_ids, tokens, temperature, top_k, top_p, uniforms, feed_rows=None):
+        """Start one decode step (one token per request, logits sampled at once) and return a
+        ticket for decode_collect. Nothing here waits for the device.
 
+        tokens: the requests' next tokens, or None: then request i takes the token that the
+        previous launch sampled in its row feed_rows[i], straight from the device, so that
+        this step can be launched before the previous one's tokens have been read.
         With use_graphs the whole step (model and sampler) is one captured HIP graph per
         (batch size, context bucket); tables and sampling options go into fixed buffers first.
-        Returns (tokens, logprobs, logits); logits stay on the device.
         """
         n = len(request_ids)
-        for rid, t in zip(request_ids, tokens):
-            if not 0 <= int(t) < self.vocab_size:
-                raise ValueError(f"request {rid!r}: token {t} outside the vocabulary of {self.vocab_size}")
+        if tokens is None:
+            if self._last_picked is None or feed_rows is None or len(feed_rows) != n:
+                raise ValueError("decode_launch without tokens needs a previous launch and its rows to take them from")
+            if any(not 0 <= int(r) < self._last_picked.shape[0] for r in feed_rows):
+                raise ValueError("decode_launch: a row to take a token from is not a row of the previous launch")
+        else:
+            for rid, t in zip(request_ids, tokens):
+                if not 0 <= int(t) < self.vocab_size:
+                    raise ValueError(f"request {rid!r}: token {t} outside the vocabulary of {self.vocab_size}")
+        for rid in request_ids:
             if self.cache.seq_len(rid) + 1 > self.max_position:
                 raise ValueError(f"request {rid!r} would pass max_position_embeddings {self.max_position}")
         graphs = self.engine_config.use_graphs and self.rt.device.type == "cuda"
@@ -153,7 +177,13 @@ class ModelRunner:
         tables = self.cache.begin_step([(rid, 1) for rid in request_ids])
         try:
             tables = self.cache.pad_tables(tables, pad)
-            batch = self.builder.build(tables, [[int(t)] for t in tokens] + [[0]] * pad, list(range(rows)))
+            host_tokens = [[0]] * rows if tokens is None else [[int(t)] for t in tokens] + [[0]] * pad
+            batch = self.builder.build(tables, host_tokens, list(range(rows)))
+            if tokens is None:
+                # after the tables' copy and before the step: the sampled tokens become the new tokens
+                self._feed_host[:n] = torch.as_tensor(list(feed_rows), dtype=torch.int64)
+                self._feed_dev[:n].copy_(self._feed_host[:n], non_blocking=True)
+                batch.token_ids[:n].copy_(self._last_picked[:, 0].index_select(0, self._feed_dev[:n]))
             # rows that only fill the batch up are chosen greedily and thrown away
             self._put_sampling(rows, list(temperature) + [0.0] * pad, list(top_k) + [0] * pad,
                                list(top_p) + [1.0] * pad, list(uniforms) + [0.0] * pad)
@@ -164,8 +194,28 @@ class ModelRunner:
                     logits, picked = self._decode_body(batch)
         finally:
             self.cache.end_step()
-        host = picked[:n].cpu()
-        return host[:, 0].tolist(), host[:, 1].contiguous().view(torch.float32).tolist(), logits[:n]
+        slot = self._launches & 1
+        self._launches += 1
+        self._last_picked = picked
+        self._picked_host[slot][:n].copy_(picked[:n], non_blocking=True)
+        if self._picked_ready[slot] is not None:
+            self._picked_ready[slot].record()
+        return (slot, n, logits[:n])
+
+    def decode_collect(self, ticket):
+        """Wait for a launched decode step; returns (tokens, logprobs) as Python lists."""
+        slot, n, _ = ticket
+        if self._picked_ready[slot] is not None:
+            self._picked_ready[slot].synchronize()
+        host = self._picked_host[slot][:n]
+        return host[:, 0].tolist(), host[:, 1].contiguous().view(torch.float32).tolist()
+
+    def decode_and_sample(self, request_ids, tokens, temperature, top_k, top_p, uniforms):
+        """decode_launch and decode_collect in one call. Returns (tokens, logprobs, logits); logits
+        stay on the device and hold until the next launch."""
+        ticket = self.decode_launch(request_ids, tokens, temperature, top_k, top_p, uniforms)
+        toks, logps = self.decode_collect(ticket)
+        return toks, logps, ticket[2]
 
     def graph_batch_size(self, n: int) -> int:
         """The batch size whose graph serves n decoding requests: n itself up to 8, then the

@@ -175,11 +175,30 @@ class Scheduler:
             take(r, self.prefill_chunk)
         return StepPlan(entries, failed)
 
+    def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
+        """The step after ``plan``, decided before plan's sampled tokens are known. That is
+        possible only when nothing but the tokens themselves is missing: plan is one token of
+        every running request and nobody waits. Requests for which plan's token is the last
+        (max_new_tokens) are left out. A request that ends on a stop sequence in ``plan`` is
+        found out only later; finish_step then skips its entry in the step returned here (the
+        token it computed is dropped, its pages go back with the request). The tokens of the
+        entries are None: they are still on the device."""
+        live = [e for e in plan.entries if not e.request.finished]
+        if self.waiting or len(live) != len(self.running):
+            return None
+        if any(len(e.tokens) != 1 or not e.sample for e in live):
+            return None
+        entries = [PlannedEntry(e.request, [None], sample=True) for e in live
+                   if len(e.request.output) + 1 < e.request.max_new]
+        return StepPlan(entries, []) if entries else None
+
     def finish_step(self, plan: StepPlan, sampled: Dict[object, Tuple[int, float]]) -> List[Request]:
         """Book the step: tokens are in the cache, sampled tokens join the outputs. Returns who finished."""
         done = []
         for e in plan.entries:
             r = e.request
+            if r.finished:                  # ended while this step, decided ahead, was already under way
+                continue
             r.num_computed += len(e.tokens)
             if not e.sample:
                 continue

@@ -109,3 +109,60 @@ def test_prepared_matrices_follow_the_tensor_not_its_address():
         del t
     rt.forget_casts()
     assert not rt._cast
+
+
+def test_steps_launched_ahead_give_the_same_generation(folder_a):
+    """With lookahead the next decode step is launched before this one's tokens are read. Requests
+    of different lengths, one that ends on a stop sequence (found out one step late: the step
+    already under way computed a token for it, which is dropped), more requests than may be live
+    at once, temperature sampling: outputs, logprobs and finish reasons equal the run without it."""
+    cfg, w = plain.read_folder(folder_a)
+    V = TINY_A["vocab_size"]
+    prompts = [tt.random_tokens(V, n, seed=30 + n) for n in (9, 3, 40, 17, 5, 64)]
+    free = plain.greedy_generate(cfg, w, prompts[0], 12)
+    params = [SamplingParams(temperature=0.0, max_new_tokens=12, stop_ids=[free[4:6]]),
+              SamplingParams(temperature=0.0, max_new_tokens=1),
+              SamplingParams(temperature=0.8, top_k=20, max_new_tokens=9, seed=5),
+              SamplingParams(temperature=0.0, max_new_tokens=2),
+              SamplingParams(temperature=1.1, top_p=0.8, max_new_tokens=15, seed=6),
+              SamplingParams(temperature=0.0, max_new_tokens=7)]
+
+    def run(lookahead, max_reside):
+        ec = EngineConfig(dtype="float32", page_size=16, max_token=1024, max_reside=max_reside, max_step_tokens=64,
+                          prefill_chunk=32, device="cpu", seed=3, lookahead=lookahead)
+        eng = Engine(runner=ModelRunner(folder_a, engine_config=ec, ops=TorchOps()))
+        out = eng.generate(prompts, params)
+        eng.runner.cache.check_invariants()
+        assert not eng.runner.cache.live and eng._in_flight is None
+        assert all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+        return [(r.output_ids, r.finish_reason, [round(x, 5) for x in r.output_logprobs]) for r in out], eng
+
+    plain_run, _ = run(False, 6)
+    ahead_run, eng = run(True, 6)
+    assert ahead_run == plain_run
+    assert plain_run[0][1] == "stop" and len(plain_run[0][0]) < 12
+    # requests wait for a slot: steps are decided ahead only now and then (other batches: logprobs to rounding)
+    waited = run(True, 2)[0]
+    assert [(o, why) for o, why, _ in waited] == [(o, why) for o, why, _ in plain_run]
+    assert all(abs(x - y) < 1e-3 for (_, _, a), (_, _, b) in zip(waited, plain_run) for x, y in zip(a, b))
+    assert eng.decode_tokens == sum(len(o) - 1 for o, _, _ in plain_run)    # a dropped token is not counted
+
+
+def test_schedule_ahead_only_when_the_tokens_are_all_that_is_missing(folder_a):
+    from return_amd.engine.scheduler import Request, Scheduler
+    runner = runner_for(folder_a, 512, max_reside=3)
+    sch = Scheduler(runner.cache, 3, 64, 32, runner.max_position)
+    a = Request("a", [1, 2, 3], SamplingParams(max_new_tokens=3))
+    b = Request("b", [4, 5], SamplingParams(max_new_tokens=2))
+    sch.add(a); sch.add(b)
+    plan = sch.schedule()                                    # both prompts whole
+    assert sch.schedule_ahead(plan) is None                  # not a decode step
+    sch.finish_step(plan, {"a": (7, 0.0), "b": (8, 0.0)})
+    for r, n in ((a, 3), (b, 2)):                            # the runner's side of the step
+        runner.cache.begin_step([(r.id, n)]); runner.cache.end_step()
+    plan = sch.schedule()
+    assert [e.tokens for e in plan.entries] == [[7], [8]]
+    ahead = sch.schedule_ahead(plan)                         # b's second token is its last: only a goes on
+    assert [e.request.id for e in ahead.entries] == ["a"] and ahead.entries[0].tokens == [None]
+    sch.add(Request("c", [9], SamplingParams(max_new_tokens=2)))
+    assert sch.schedule_ahead(plan) is None                  # somebody waits: the next step is not only decoding
