@@ -97,3 +97,35 @@ def test_generation_with_graphs(folder_b):
                      max_step_tokens=64, prefill_chunk=24, use_graphs=use_graphs)
         outs.append([r.output_ids for r in eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=20))])
     assert outs[0] == outs[1]
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_steps_launched_ahead_on_the_device(folder_b, dtype, use_graphs):
+    """The next decode step is launched before this one's tokens are read and takes them over on
+    the device: outputs, logprobs and finish reasons equal the run that waits for every step.
+    Lengths differ, one request ends on a stop sequence that is found out a step late, eleven
+    requests make the graph of sixteen rows shrink to that of eight and below."""
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    V = TINY_B["vocab_size"]
+    prompts = [tt.random_tokens(V, n, seed=50 + n) for n in (9, 3, 40, 17, 5, 64, 2, 33, 12, 7, 21)]
+    news = [12, 1, 9, 2, 15, 7, 30, 4, 11, 26, 5]
+
+    def run(lookahead, stops):
+        eng = Engine(folder_b, dtype=dtype, page_size=16, max_token=4096, max_reside=11, max_step_tokens=128,
+                     prefill_chunk=64, use_graphs=use_graphs, lookahead=lookahead, seed=4)
+        params = [SamplingParams(temperature=0.0 if i % 3 else 0.9, top_k=0 if i % 2 else 30, max_new_tokens=n,
+                                 seed=i, stop_ids=stops if i == 6 else [])
+                  for i, n in enumerate(news)]
+        out = eng.generate(prompts, params)
+        eng.runner.cache.check_invariants()
+        assert not eng.runner.cache.live and all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+        return [(r.output_ids, r.finish_reason, r.output_logprobs) for r in out]
+
+    free = run(False, [])
+    stop = [free[6][0][9:11]]                     # two tokens that request 6 will write
+    want, got = run(False, stop), run(True, stop)
+    assert got == want
+    assert want[6][1] == "stop" and len(want[6][0]) < 30
+    assert [len(o) for o, _, _ in want][:6] == news[:6]
