@@ -1,7 +1,9 @@
 // y = x @ W^T for row-major x [M, K] and W [N, K] (the nn.Linear layout of the reference,
 // rollout/monkey_patch/qwen3.py:21). This file holds the plain tiled kernel: products and
 // sums in true 32-bit FMA, K walked in order, so a row's result does not depend on M.
-// It is the only matrix product of the float32 path and the fallback of the bfloat16 path.
+// It is the matrix product of the float32 path and the fallback of the bfloat16 path. For up to
+// 16 rows of x in float32 (decoding) there is a second kernel that streams W once with 16-byte
+// loads; it sums a row's products in another order than the tiled kernel, 32-bit all the same.
 #include "common.h"
 
 #define BM 64
@@ -65,6 +67,64 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TI* __restrict__ A,
     }
 }
 
+// ------------------------------------------------------------------ few rows, float32
+// y[m, n] = sum_k x[m, k] W[n, k] for M <= MR rows, all float32, K % 4 == 0. A workgroup of four
+// waves takes 16 rows of W, four per wave; x goes through LDS in blocks of 512 columns for all
+// four waves; a lane multiplies the four floats at k = 4 lane (+256) of its rows of W with the same
+// four floats of every row of x, and the lanes' sums are added at the end (lane order, fixed).
+typedef float gv_f4 __attribute__((ext_vector_type(4)));
+#define GV_KC 512
+template <int MR>
+__global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__ x, const float* __restrict__ W,
+                                                       float* __restrict__ y, int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) float x_s[MR][GV_KC];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int n0 = (blockIdx.x * 4 + wave) * 4;
+    const float* wr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) wr[r] = W + (size_t)min(n0 + r, N - 1) * K;      // clamped: loads stay inside W
+    float acc[4][MR];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
+    const gv_f4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += GV_KC) {
+        __syncthreads();                                     // every wave has left the last block of x
+        for (int e = tid; e < MR * (GV_KC / 4); e += 256) {
+            const int m = e / (GV_KC / 4), k = k0 + 4 * (e % (GV_KC / 4));
+            *reinterpret_cast<gv_f4*>(&x_s[m][k - k0]) =
+                (m < M && k < K) ? *reinterpret_cast<const gv_f4*>(x + (size_t)m * K + k) : zero;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < GV_KC / 256; ++h) {
+            const int kl = 256 * h + 4 * lane, k = k0 + kl;
+            gv_f4 w[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) w[r] = k < K ? *reinterpret_cast<const gv_f4*>(wr[r] + k) : zero;
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                const gv_f4 xv = *reinterpret_cast<const gv_f4*>(&x_s[m][kl]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[r][m] = fmaf(w[r][0], xv[0], acc[r][m]);
+                    acc[r][m] = fmaf(w[r][1], xv[1], acc[r][m]);
+                    acc[r][m] = fmaf(w[r][2], xv[2], acc[r][m]);
+                    acc[r][m] = fmaf(w[r][3], xv[3], acc[r][m]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const float s = wave_sum(acc[r][m]);
+            if (lane == 0 && m < M && n0 + r < N) y[(size_t)m * N + n0 + r] = s;
+        }
+}
+
 // in_dtype / out_dtype: RA_DTYPE_F32 or RA_DTYPE_BF16 (x and W share in_dtype)
 extern "C" int ra_gemm_nt(const void* A, const void* W, void* C, int M, int N, int K, int in_dtype,
                           int out_dtype, void* stream) {
@@ -72,6 +132,17 @@ extern "C" int ra_gemm_nt(const void* A, const void* W, void* C, int M, int N, i
     if (K <= 0) return RA_ERR_ARG;
     dim3 block(256), grid((N + BN - 1) / BN, (M + BM - 1) / BM);
     hipStream_t s = (hipStream_t)stream;
+    if (in_dtype == RA_DTYPE_F32 && out_dtype == RA_DTYPE_F32 && M <= 16 && K % 4 == 0) {
+        const dim3 g16((N + 15) / 16);
+        const float *xa = (const float*)A, *wa = (const float*)W;
+        float* ya = (float*)C;
+        if (M <= 1) hipLaunchKernelGGL(gemv_f32_kernel<1>, g16, block, 0, s, xa, wa, ya, M, N, K);
+        else if (M <= 2) hipLaunchKernelGGL(gemv_f32_kernel<2>, g16, block, 0, s, xa, wa, ya, M, N, K);
+        else if (M <= 4) hipLaunchKernelGGL(gemv_f32_kernel<4>, g16, block, 0, s, xa, wa, ya, M, N, K);
+        else if (M <= 8) hipLaunchKernelGGL(gemv_f32_kernel<8>, g16, block, 0, s, xa, wa, ya, M, N, K);
+        else hipLaunchKernelGGL(gemv_f32_kernel<16>, g16, block, 0, s, xa, wa, ya, M, N, K);
+        return ra_launch_status();
+    }
     if (in_dtype == RA_DTYPE_F32 && out_dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL((gemm_nt_kernel<float, float>), grid, block, 0, s, (const float*)A,
                            (const float*)W, (float*)C, M, N, K);

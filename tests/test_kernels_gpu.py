@@ -239,6 +239,18 @@ def test_tiled_mfma_product(ops, out_dtype, M, N, K):
         torch.testing.assert_close(y.double(), want, atol=3e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 8, 9, 16, 17])
+@pytest.mark.parametrize("N,K", [(331, 120), (48, 1000), (1000, 4), (70, 4096), (16, 516)])
+def test_linear_float32_few_rows(ops, M, N, K):
+    """float32 rows times float32 weights: up to 16 rows go to the kernel that streams W once,
+    more to the tiled kernel; both are plain 32-bit sums."""
+    x = rnd(M, K, seed=91)
+    w = rnd(N, K, seed=92, scale=0.3)
+    y = ops.linear(x, w)
+    assert y.dtype == torch.float32
+    torch.testing.assert_close(y.double(), x.double() @ w.double().t(), atol=2e-6 * K ** 0.5 + 1e-6, rtol=1e-5)
+
+
 def test_linear_fp32_is_true_fp32(ops):
     """Inputs 1 + 2^-12 round to 1 in bf16 and tf32; a true 32-bit product keeps the 2^-11 per term."""
     K = 64
