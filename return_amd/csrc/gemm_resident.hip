@@ -5,7 +5,7 @@
 //
 // A workgroup first copies x into LDS, [8 or 16][K + 8] (rows shifted by four banks). Then it
 // walks over tiles of 16 rows of W (tile = blockIdx.x, += gridDim.x): its waves split K in
-// blocks of 256, W is the A operand of MFMA 16x16x32 bf16 read straight from memory (lane
+// blocks of 256 (128 when GATED), W is the A operand of MFMA 16x16x32 bf16 read straight from memory (lane
 // (n, g): 16 bytes of row n at k0 + 8g), x the B operand read from LDS, and the waves' partial
 // tiles are added through LDS in wave order (one barrier, then every thread adds one element). x is read from the cache once per workgroup
 // instead of once per tile, and the loop issues no loads but W's.
@@ -19,7 +19,6 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 #define RG_UNROLL 8
-#define RG_KB (32 * RG_UNROLL)
 
 template <int WAVES, int MP, bool GATED, typename TO>
 __global__ __launch_bounds__(WAVES * 64) void gemm_resident_kernel(
@@ -33,6 +32,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_resident_kernel(
     float* red = reinterpret_cast<float*>(lds_raw + (size_t)MP * XS * 2);   // [WAVES][NG][16][MP + 1]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // The blocks of W that this wave multiplies, in order: for every tile of the workgroup its k-blocks
+    // wave, wave + WAVES, ... The next block is asked for before this one is multiplied, the first one
+    // before x is copied, so that W keeps streaming through the copy and through the tiles' ends.
+    constexpr int U = GATED ? RG_UNROLL / 2 : RG_UNROLL;    // MFMA steps per block (two operands each when GATED)
+    constexpr int KB = 32 * U;
+    const int n_kb = K > wave * KB ? (K - wave * KB + WAVES * KB - 1) / (WAVES * KB) : 0;
+    bf16x8_t a_next[NG][U];
+    int next_tile = blockIdx.x, next_j = 0;
+    auto fetch = [&]() {
+        if (next_tile >= n_tiles || n_kb == 0) return;
+        const int row = min(next_tile * 16 + n, N - 1);     // clamped: loads stay inside W
+        const bf16* wp = W + (size_t)row * K + g * 8;
+        const bf16* wp_up = wp + (size_t)N * K;             // GATED: the up row of the same column
+        const int kb = (wave + next_j * WAVES) * KB;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = kb + u * 32;
+            const bool in = k + g * 8 < K;                  // K % 8 == 0: a lane's 8 are in or out together
+            a_next[0][u] = in ? *reinterpret_cast<const bf16x8_t*>(wp + k) : zero;
+            if constexpr (GATED) a_next[1][u] = in ? *reinterpret_cast<const bf16x8_t*>(wp_up + k) : zero;
+        }
+    };
+    fetch();
 
     // ---- x into LDS, rows beyond M as zeros
     {
@@ -48,26 +71,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_resident_kernel(
 
     for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int n0 = tile * 16;
-        const int row = min(n0 + n, N - 1);                 // clamped: loads stay inside W
-        const bf16* wp = W + (size_t)row * K + g * 8;
-        const bf16* wp_up = wp + (size_t)N * K;               // GATED: the up row of the same column
         float4_t c[NG][MB];
 #pragma unroll
         for (int z = 0; z < NG; ++z)
 #pragma unroll
             for (int b = 0; b < MB; ++b) c[z][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-        for (int kb = wave * RG_KB; kb < K; kb += WAVES * RG_KB) {
-            bf16x8_t a[NG][RG_UNROLL];
+        for (int j = 0; j < n_kb; ++j) {
+            bf16x8_t a[NG][U];
 #pragma unroll
-            for (int u = 0; u < RG_UNROLL; ++u) {
-                const int k = kb + u * 32;
-                const bool in = k + g * 8 < K;               // K % 8 == 0: a lane's 8 are in or out together
-                a[0][u] = in ? *reinterpret_cast<const bf16x8_t*>(wp + k) : zero;
-                if constexpr (GATED) a[1][u] = in ? *reinterpret_cast<const bf16x8_t*>(wp_up + k) : zero;
+            for (int z = 0; z < NG; ++z)
+#pragma unroll
+                for (int u = 0; u < U; ++u) a[z][u] = a_next[z][u];
+            if (j + 1 < n_kb) {
+                next_j = j + 1;
+            } else {
+                next_tile = tile + gridDim.x;
+                next_j = 0;
             }
+            fetch();
+            const int kb = (wave + j * WAVES) * KB;
 #pragma unroll
-            for (int u = 0; u < RG_UNROLL; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int k = kb + u * 32 + g * 8;
                 const bool in = k < K;
 #pragma unroll

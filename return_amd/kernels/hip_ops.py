@@ -114,12 +114,12 @@ class HipOps:
 
     def use_resident(self, M, N, K, gated):
         """Whether the product with x resident in LDS beats the skinny product for x [M, K] and
-        N result columns (measured on MI355X): from two rows on, when every workgroup gets
-        several tiles of 16 columns; one row and few tiles are the skinny product's."""
+        N result columns (measured on MI355X): when there are tiles of 16 columns enough for
+        every workgroup (two per CU); few tiles are the skinny product's."""
         if not self.lib.ra_gemm_resident_fits(M, K, 1 if gated else 0):
             return False
         tiles = -(-N // 16)
-        if 2 <= M <= 8:
+        if 1 <= M <= 8:
             return tiles >= 384
         return M > 8 and tiles >= 2048
 
