@@ -38,7 +38,9 @@ PAGE = 16
 PREFILL_TOKENS = 2048
 
 
-def build_runner(layers, dtype, max_reside, seed=0, use_graphs=True):
+def build_runner(layers, dtype, max_reside, seed=0, use_graphs=True, raw=None, std=0.02, **engine_options):
+    """A runner with random weights made on the GPU. raw: config.json keys (default: the 8B shape
+    with ``layers`` layers); engine_options override the engine configuration of the headline run."""
     import torch
     import return_amd.models  # noqa: F401
     from return_amd.config import EngineConfig, Qwen3Config
@@ -46,15 +48,16 @@ def build_runner(layers, dtype, max_reside, seed=0, use_graphs=True):
     from return_amd.config import lookup_architecture
     from return_amd.weights import random_weights
 
-    raw = dict(QWEN3_8B, num_hidden_layers=layers)
+    raw = dict(QWEN3_8B, num_hidden_layers=layers) if raw is None else raw
     cfg = Qwen3Config.from_dict(raw)
     _, build_spec = lookup_architecture(cfg.architecture)
-    weights = random_weights(build_spec(cfg), seed=seed, std=0.02, dtype=dtype, device="cuda:0",
+    weights = random_weights(build_spec(cfg), seed=seed, std=std, dtype=dtype, device="cuda:0",
                              generator_device="cuda:0")
-    ec = EngineConfig(dtype=dtype, page_size=PAGE, max_token=max_reside * MAX_CONTEXT,
-                      max_reside=max_reside, max_step_tokens=max(PREFILL_TOKENS, max_reside),
-                      prefill_chunk=PREFILL_TOKENS, use_graphs=use_graphs)
-    runner = ModelRunner(config=cfg, weights=weights, engine_config=ec)
+    options = dict(dtype=dtype, page_size=PAGE, max_token=max_reside * MAX_CONTEXT,
+                   max_reside=max_reside, max_step_tokens=max(PREFILL_TOKENS, max_reside),
+                   prefill_chunk=PREFILL_TOKENS, use_graphs=use_graphs)
+    options.update(engine_options)
+    runner = ModelRunner(config=cfg, weights=weights, engine_config=EngineConfig(**options))
     del weights
     torch.cuda.empty_cache()
     return cfg, runner
@@ -134,8 +137,120 @@ def release(runner, ids):
         runner.free_request(rid)
 
 
+# BASELINE.json configs[3] and configs[4]: the other two shapes, with the workloads named there
+QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64,
+                 intermediate_size=25600)
+
+
+def shape_of(cfg, **more):
+    d = {"hidden": cfg.hidden_size, "layers": cfg.num_hidden_layers, "heads": cfg.num_attention_heads,
+         "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size,
+         "vocab": cfg.vocab_size, "page_size": PAGE, "parallelism": "single GPU"}
+    d.update(more)
+    return d
+
+
+def continuous_4b(args):
+    """Continuous batching on the Qwen3-4B shape: 128 requests, prompts of 64 to 4,096 tokens and
+    32 to 512 new tokens each (uniform), prompts in portions of 512 beside the decoded tokens,
+    through Engine.generate. value: generated tokens a second over the whole run."""
+    import random
+    import torch
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    n = args.batch if args.batch != 8 else 128
+    cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_4B, use_graphs=not args.no_graphs,
+                               max_token=n * 4608, max_step_tokens=512 + n, prefill_chunk=512)
+    eng = Engine(runner=runner)
+    rnd = random.Random(0)
+    prompts = [[rnd.randrange(cfg.vocab_size) for _ in range(rnd.randint(64, 4096))] for _ in range(n)]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=rnd.randint(32, 512)) for _ in range(n)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = eng.generate(prompts, params)
+    torch.cuda.synchronize()
+    secs = time.perf_counter() - t0
+    if any(r.num_tokens != p.max_new_tokens for r, p in zip(out, params)):
+        raise RuntimeError("a request ended early")
+    runner.cache.check_invariants()
+    made, read = sum(r.num_tokens for r in out), sum(map(len, prompts))
+    flops = 2.0 * (read + made) * (weight_bytes(cfg, 1) - cfg.vocab_size * cfg.hidden_size)
+    return {"metric": "generated tok/s, continuous batching (Qwen3-4B shape, random weights)",
+            "value": round(made / secs, 1), "unit": "tok/s", "n_gpus": 1, "steps": eng.steps, "warmup": 0,
+            "ms_per_step": round(secs / eng.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": shape_of(cfg, model="Qwen3-4B shape", global_batch=n, prompt_tokens=read, new_tokens=made,
+                               prefill_chunk=512, max_context=4608, hip_graphs=not args.no_graphs,
+                               weights="random N(0,0.02)"),
+            "seconds": round(secs, 3), "prompt_tok_s": round(read / secs, 1),
+            "linear_flops_frac": round(flops / secs / PEAK_FLOPS[args.dtype], 4)}
+
+
+def long_32b(args):
+    """Long contexts on the Qwen3-32B shape: 16 prompts of 8,192 tokens (one portion each), then
+    decoding at batch 16, then one prompt of 32,768 tokens in portions of 8,192. value: decoded
+    tokens a second."""
+    import random
+    import torch
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    elt = 2 if args.dtype == "bfloat16" else 4
+    n, ctx, new, long_ctx = 16, 8192, max(2, args.steps), 32768
+    cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_32B, std=0.01, use_graphs=not args.no_graphs,
+                               max_token=n * (ctx + 512) + long_ctx, max_step_tokens=ctx, prefill_chunk=ctx)
+    eng = Engine(runner=runner)
+    rnd = random.Random(1)
+    prompts = [[rnd.randrange(cfg.vocab_size) for _ in range(ctx)] for _ in range(n)]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=new)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reqs = [eng.submit(p, sp) for p in prompts]
+    while any(not r.output for r in reqs):
+        eng.step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    d0, n0 = eng.decode_tokens, eng.steps
+    while eng.scheduler.has_work():
+        eng.step()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    runner.cache.check_invariants()
+    steps, made = eng.steps - n0, eng.decode_tokens - d0
+    ms_step = (t2 - t1) / steps * 1e3
+    step_bytes = weight_bytes(cfg, elt) + n * (ctx + new / 2.0) * kv_bytes_per_token(cfg, elt)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    long_prompt = [rnd.randrange(cfg.vocab_size) for _ in range(long_ctx)]
+    best = None
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        eng.generate([long_prompt], SamplingParams(temperature=0.0, max_new_tokens=1))
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t3
+        best = dt if best is None else min(best, dt)
+
+    def pre(tokens, secs, count):
+        f = count * prefill_flops(cfg, tokens)
+        return {"value": round(count * tokens / secs, 1), "tokens": count * tokens, "ms": round(secs * 1e3, 1),
+                "frac": round(f / secs / PEAK_FLOPS[args.dtype], 4)}
+    return {"metric": "decode tok/s at batch 16, 8,192-token prompts (Qwen3-32B shape, random weights)",
+            "value": round(made / (t2 - t1), 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+            "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": shape_of(cfg, model="Qwen3-32B shape", global_batch=n, seq_len=ctx, new_tokens=new,
+                               long_prompt=long_ctx, prefill_chunk=ctx, hip_graphs=not args.no_graphs,
+                               weights="random N(0,0.01)"),
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(achieved / PEAK_HBM_GBS, 4)},
+            "prefill": pre(ctx, t1 - t0, n), "prefill_long": pre(long_ctx, best, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="decode_8b", choices=["decode_8b", "continuous_4b", "long_32b"],
+                    help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
+                         "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
@@ -153,6 +268,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible")
         return 1
+    if args.workload != "decode_8b":
+        print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b}[args.workload](args)))
+        return 0
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),
                                use_graphs=not args.no_graphs)

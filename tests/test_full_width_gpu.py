@@ -1,0 +1,95 @@
+"""The engine at the layer sizes of Qwen3-8B (width 4096, 32 query heads on 8 kv heads of 128,
+intermediate 12288; two layers and a shorter vocabulary keep it quick): the products, attention
+kernels and graph paths that serving at that shape takes, under every way of cutting the work,
+against the plain implementation. The tiny configurations never reach these kernels' fast paths
+(x resident in LDS, the library's products, head size 128 with four query heads a kv head)."""
+import pytest
+import torch
+
+from tests import trace_tools as tt
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+WIDE = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=32003, hidden_size=4096,
+    num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+    intermediate_size=12288, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1e6,
+    tie_word_embeddings=False)
+LENGTHS = {"a": 5, "b": 17, "c": 700, "d": 100, "e": 64, "f": 150, "g": 1, "h": 47}
+# float32: the bounds of the tiny configurations' replay. bfloat16: every product's result, the cache
+# and the attention's probabilities are rounded to 8 bits of mantissa, which leaves noise of about
+# 1.2 % of a row's norm (bounded below at 2 %, the reference's own bound); the logits' standard
+# deviation here is 1.3, so one logit is off by 0.016 (one sigma), and the largest of the 35 million
+# compared ones by six sigma.
+TOL = {"float32": dict(atol=2e-4, rtol=2e-4), "bfloat16": dict(atol=1e-1, rtol=5e-2)}
+
+
+@pytest.fixture(scope="module")
+def wide(tmp_path_factory):
+    from tests.conftest import make_folder
+    folder = make_folder(tmp_path_factory, "wide", WIDE, dict(seed=5, std=0.02, embedding_std=0.02, norm_jitter=0.01))
+    reqs = {rid: tt.random_tokens(WIDE["vocab_size"], n, seed=ord(rid)) for rid, n in LENGTHS.items()}
+    cfg, w = plain.read_folder(folder)
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    return folder, reqs, want
+
+
+def runner_for(folder, dtype, max_tokens, **kw):
+    from return_amd.config import EngineConfig
+    from return_amd.engine import ModelRunner
+    ec = EngineConfig(dtype=dtype, page_size=16, max_token=max_tokens, max_reside=4,
+                      max_step_tokens=max(max_tokens, 4), prefill_chunk=max_tokens, **kw)
+    return ModelRunner(folder, engine_config=ec)
+
+
+def compare(got, want, reqs, dtype):
+    worst, worst_rel = 0.0, 0.0
+    for rid, toks in reqs.items():
+        for p in range(len(toks)):
+            a, b = got[(rid, p)], want[rid][p]
+            worst = max(worst, (a - b).abs().max().item())
+            worst_rel = max(worst_rel, ((a - b).norm() / b.norm()).item())
+            try:
+                torch.testing.assert_close(a, b, **TOL[dtype])
+            except AssertionError as e:
+                raise AssertionError(f"request {rid} position {p} (first wrong place): {e}") from None
+    return worst, worst_rel
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail_decoded", "portions", "mixed"])
+def test_full_width_replay(wide, dtype, cut):
+    folder, reqs, want = wide
+    steps = {"whole": tt.whole, "tail_decoded": tt.tail_decoded, "portions": tt.portions,
+             "mixed": tt.mixed}[cut](reqs)
+    runner = runner_for(folder, dtype, tt.peak_tokens(steps))
+    got = tt.run_in_process(runner, steps)
+    worst, rel = compare(got, want, reqs, dtype)
+    print(f"full width {dtype} {cut}: largest difference {worst:.2e}, largest relative L2 {rel:.2e}")
+    # the reference's own bound on a bf16 kernel against 32-bit: relative L2 of 2e-2 (rollout/utils/test_prefill_fwd_bwd.py:117)
+    assert rel < (2e-2 if dtype == "bfloat16" else 1e-4)
+    assert not runner.cache.live
+
+
+def test_full_width_generation_through_graphs(wide):
+    """Greedy generation in bfloat16 through the entry point, graphs and steps launched ahead on,
+    four requests at once: every generated token is the 32-bit plain implementation's first or
+    second choice at its place given the same prefix, and its logprob agrees."""
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    folder, reqs, _ = wide
+    cfg, w = plain.read_folder(folder)
+    prompts = [reqs[r] for r in ("b", "d", "e", "h")]
+    eng = Engine(folder, dtype="bfloat16", page_size=16, max_token=2048, max_reside=4, max_step_tokens=256,
+                 prefill_chunk=96)
+    out = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=12))
+    for p, r in zip(prompts, out):
+        assert r.num_tokens == 12
+        rows = plain.logits(cfg, w, list(p) + r.output_ids[:-1])[len(p) - 1:]
+        for i, tok in enumerate(r.output_ids):
+            top2 = rows[i].topk(2)
+            assert tok in top2.indices.tolist(), f"token {i}: {tok} is not among the plain top two {top2.indices.tolist()}"
+            if tok != int(top2.indices[0]):           # a near tie that bfloat16 may decide the other way
+                assert float(top2.values[0] - top2.values[1]) < 0.1
+            assert abs(r.output_logprobs[i] - plain.chosen_logprob(rows[i], tok)) < 0.1
