@@ -22,7 +22,8 @@
 //          l%4 of the 8 bytes addressed by lanes l/4, l/4+4, l/4+8, l/4+12), and P goes from
 //          the softmax registers straight into the B operand because the contraction runs over
 //          keys in the order the lanes already hold them (k-slot (g, e) of a 32-key block is
-//          key 16*(e/4) + 4g + e%4). The cost does not depend on how many heads share a kv head.
+//          key 16*(e/4) + 4g + e%4). The cost does not depend on how many heads share a kv head,
+//          up to 16; a larger group takes one wave per 16 heads, which read the same keys.
 // BUILD-VARIANTS: DEC_PART=0 DEC_PART=1 DEC_PART=2 DEC_PART=3 DEC_API=1
 // (each DEC_PART instantiates four head sizes; DEC_API holds the entry point and the merge)
 #include "common.h"
@@ -37,7 +38,7 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 typedef short4_t __attribute__((address_space(3))) * lds_short4_ptr;
 
 #define DEC_CHUNK 64          // keys per pass of a wave
-#define DEC_MAX_GROUP 16      // query heads per kv head (columns of the MFMA tile)
+#define DEC_MAX_GROUP 16      // query heads a wave takes (columns of the MFMA tile); larger groups take several waves
 
 struct DecodeRange {
     int lo, hi;               // key positions of this split, inclusive; lo > hi: empty
@@ -81,10 +82,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
 
     __shared__ __attribute__((aligned(16))) uint16_t v_s[DEC_CHUNK * VS];
 
-    const int di = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
+    // blockIdx.y: kv head and, when more than 16 query heads share it, which 16 of them
+    const int group = Hq / Hkv, blocks = (group + DEC_MAX_GROUP - 1) / DEC_MAX_GROUP;
+    const int di = blockIdx.x, kvh = blockIdx.y / blocks, hb = blockIdx.y - kvh * blocks, sp = blockIdx.z;
     const int seg = seg_ids ? seg_ids[di] : di;
     const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
-    const int G = Hq / Hkv;
+    const int h0 = kvh * group + hb * DEC_MAX_GROUP;             // first query head of this wave
+    const int G = min(DEC_MAX_GROUP, group - hb * DEC_MAX_GROUP);  // and how many it has
     const int t = cu_q[seg];
     const int pos_q = q_start[seg];
     const int start = kv_start[seg];
@@ -93,12 +97,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
     const int* pt = page_table + cu_pages[seg];
     const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
 
-    // query operand: lane (n, g) holds head kvh*G+n, d = 32j + 8g .. +7 (and D-16+8g.. for the tail)
+    // query operand: lane (n, g) holds head h0+n, d = 32j + 8g .. +7 (and D-16+8g.. for the tail)
     const bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8_t bq[D32 > 0 ? D32 : 1];
     bf16x8_t bq_tail = z8;
     {
-        const bf16* qp = q + ((size_t)t * Hq + (size_t)kvh * G + (n < G ? n : 0)) * D;
+        const bf16* qp = q + ((size_t)t * Hq + h0 + (n < G ? n : 0)) * D;
 #pragma unroll
         for (int j = 0; j < D32; ++j) {
             bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(qp + 32 * j + 8 * g);
@@ -224,11 +228,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
 
     // ---- partial results of this split: lane (n, g) holds head n, columns 16dt + 4g .. +3
     if (n < G) {
-        float* pa = part_acc + (((size_t)di * Hq + (size_t)kvh * G + n) * max_splits + sp) * D;
+        float* pa = part_acc + (((size_t)di * Hq + h0 + n) * max_splits + sp) * D;
 #pragma unroll
         for (int dt = 0; dt < D16; ++dt) *reinterpret_cast<float4_t*>(pa + dt * 16 + 4 * g) = acc[dt];
         if (g == 0) {
-            float* pm = part_ml + (((size_t)di * Hq + (size_t)kvh * G + n) * max_splits + sp) * 2;
+            float* pm = part_ml + (((size_t)di * Hq + h0 + n) * max_splits + sp) * 2;
             pm[0] = m_run;
             pm[1] = l_run;
         }
@@ -315,12 +319,13 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
                                         float scale, int window, int split_tokens, int max_splits,
                                         void* stream) {
     if (n_dec <= 0) return RA_OK;
-    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || Hq / Hkv > DEC_MAX_GROUP ||
-        split_tokens <= 0 || split_tokens % DEC_CHUNK != 0 || max_splits <= 0 || max_splits > 65535 ||
-        Hkv > 65535 || P <= 0)
+    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 ||
+        split_tokens <= 0 || split_tokens % DEC_CHUNK != 0 || max_splits <= 0 || max_splits > 65535 || P <= 0)
         return RA_ERR_ARG;
+    const int head_blocks = Hkv * ((Hq / Hkv + DEC_MAX_GROUP - 1) / DEC_MAX_GROUP);
+    if (head_blocks > 65535) return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid(n_dec, Hkv, max_splits);
+    dim3 grid(n_dec, head_blocks, max_splits);
     const bf16* qq = (const bf16*)q;
     const bf16* kp = (const bf16*)k_pool;
     const bf16* vp = (const bf16*)v_pool;

@@ -352,8 +352,7 @@ class HipOps:
         P = k_pool.shape[1]
         window = int(window)
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
-        fast_decode = (q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
-                       and n_q // n_kv <= 16)
+        fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
         if fast_decode:
             longest = step.max_decode_seq_len
             S = self.decode_split_tokens

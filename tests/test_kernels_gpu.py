@@ -311,6 +311,8 @@ ATTN_CASES = [
     (6, 2, 32, 8, [(1, 400), (1, 77), (5, 70), (1, 3)], 70),
     (4, 4, 256, 16, [(1, 199)], 0),
     (24, 1, 64, 16, [(1, 100)], 0),
+    (40, 2, 128, 16, [(1, 300), (9, 20), (1, 64), (1, 0)], 0),     # 20 heads a kv head: two waves of 16 and 4
+    (33, 1, 48, 8, [(1, 77), (1, 200)], 50),
 ]
 
 
@@ -363,8 +365,9 @@ def test_prefill_attention_every_head_size(ops, ref, D, key_split, monkeypatch):
 
 @pytest.mark.parametrize("D", list(range(16, 257, 16)))
 def test_decode_attention_every_head_size(ops, ref, D):
-    """The bfloat16 decode kernel at every head size it takes, grouped and ungrouped."""
-    for Hq, Hkv in ((4, 1), (3, 3), (16, 2)):
+    """The bfloat16 decode kernel at every head size it takes, grouped, ungrouped and with more
+    query heads to a kv head than one wave takes."""
+    for Hq, Hkv in ((4, 1), (3, 3), (16, 2), (34, 2)):
         P = 16
         segs = [(1, 150), (1, 1), (1, 64)]
         need = [-(-(a + b) // P) for b, a in segs]

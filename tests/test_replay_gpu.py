@@ -103,7 +103,7 @@ def test_long_decoding(folder_b):
 ODD = [
     # head size, heads, kv heads, width, intermediate, vocabulary, layers, page, tied
     (240, 6, 3, 100, 100, 331, 2, 4, True),       # width no multiple of 8: the plain product; a page of 4
-    (16, 60, 3, 96, 328, 1000, 2, 8, True),       # 20 query heads to a kv head: beyond the decode kernel's 16
+    (16, 60, 3, 96, 328, 1000, 2, 8, True),       # 20 query heads to a kv head: two waves of the decode kernel
     (80, 7, 1, 100, 48, 1000, 1, 32, False),      # 7 heads on one kv head, head size 80
     (256, 5, 5, 136, 100, 97, 2, 48, False),      # the largest head size, a page of 48
 ]
