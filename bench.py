@@ -323,7 +323,7 @@ def main():
                    "intermediate": cfg.intermediate_size, "vocab": V, "global_batch": args.batch,
                    "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": PAGE,
                    "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs,
+                   "hip_graphs": not args.no_graphs, "tuned_products": True,
                    "weights": "random N(0,0.02)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},

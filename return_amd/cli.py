@@ -58,7 +58,8 @@ def cmd_generate(args) -> int:
     parsed = [parse_request(r, i) for i, r in enumerate(raws)]
     engine = Engine(args.model, max_token=args.max_token, max_reside=args.max_reside, dtype=args.dtype,
                     page_size=args.page_size, seed=args.seed, max_step_tokens=args.max_step_tokens,
-                    prefill_chunk=args.prefill_chunk, use_graphs=not args.no_graphs)
+                    prefill_chunk=args.prefill_chunk, use_graphs=not args.no_graphs,
+                    tune_products=not args.no_tune)
     results = engine.generate([p for _, p, _ in parsed], [sp for _, _, sp in parsed])
     for (sid, _, _), r in zip(parsed, results):
         out = {"session_id": sid, "output_ids": r.output_ids, "output_logprobs": r.output_logprobs,
@@ -97,6 +98,8 @@ def main(argv=None) -> int:
     g.add_argument("--seed", type=int, default=0)
     g.add_argument("--no-graphs", action="store_true",
                    help="launch every kernel of a decode step from the host instead of replaying HIP graphs")
+    g.add_argument("--no-tune", action="store_true",
+                   help="choose the kernel of every projection by rule instead of measuring at load")
     g.add_argument("--requests", help="file of JSON lines (or - for standard input), one request each")
     g.add_argument("--prompt-ids", help="one prompt as comma-separated token ids")
     g.add_argument("--max-new-tokens", type=int, default=32)

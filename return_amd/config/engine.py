@@ -20,6 +20,7 @@ class EngineConfig:
     prefill_chunk: int = 8192          # longest portion of one prompt in one step
     use_graphs: bool = True            # replay decode-only steps from captured HIP graphs (USE_CUDA_GRAPH of the reference)
     lookahead: bool = True             # launch the next decode step before this one's tokens are read
+    tune_products: bool = True         # measure at load which kernel forms each projection fastest at few rows
     seed: int = 0                      # base seed of the sampling streams
     device: str = "cuda:0"
 

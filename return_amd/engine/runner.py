@@ -56,6 +56,8 @@ class ModelRunner:
             weights = load_weights(model_dir, self.spec, device=self.rt.device)
         self.model = Decoder(self.spec, weights, self.rt)
         del weights
+        if ec.tune_products and self.rt.dtype == torch.bfloat16 and hasattr(self.rt.ops, "tune_products"):
+            self.rt.ops.tune_products(self.rt.products, max_rows=ec.max_reside)
         self.cache = CacheManager(self.model.cache_layers(), ec.page_size, ec.max_token,
                                   ec.max_reside, self.rt.dtype, self.rt.device)
         self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device)

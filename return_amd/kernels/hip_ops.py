@@ -80,6 +80,11 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+# One plan per process: every engine in it forms a product of a given shape the same way.
+_PRODUCT_PLAN = {}
+_PRODUCTS_MEASURED = set()
+
+
 class HipOps:
     def __init__(self, device="cuda:0"):
         self.device = torch.device(device)
@@ -101,6 +106,8 @@ class HipOps:
             self._library_fp32_out = torch.mm(a, a.t(), out_dtype=torch.float32).dtype == torch.float32
         except (TypeError, RuntimeError):
             self._library_fp32_out = False
+        self.product_plan = _PRODUCT_PLAN    # (row step, N, K, gated, result dtype) -> way, where measured faster than the rule
+        self._tuned = _PRODUCTS_MEASURED
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -279,6 +286,62 @@ class HipOps:
                     "silu_mul")
 
     # ------------------------------------------------------------------ matrix products
+    # Ways to form y = x @ w^T from bfloat16 operands. Which is fastest depends on the shape in ways no
+    # rule captures (the library streams one weight at 5.6 TB/s and the next at 2): route_* give the
+    # rule's choice, tune_products replaces it where a measurement at load time says otherwise.
+    ROW_STEPS = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64)     # row counts at which products are measured
+
+    def _rows_step(self, M):
+        for r in self.ROW_STEPS:
+            if M <= r:
+                return r
+        return 0                                          # more rows than are ever measured: the library
+
+    def route_linear(self, M, N, K, out_dtype):
+        """How linear() forms a bfloat16 product of M rows: the measured choice if there is one, else the rule."""
+        hit = self.product_plan.get((self._rows_step(M), N, K, False, out_dtype))
+        if hit is not None:
+            return hit
+        if out_dtype in (torch.bfloat16, torch.float32) and self.use_resident(M, N, K, False):
+            return "resident512" if M <= 8 else "resident256"
+        if self.use_skinny(M, N, K, out_dtype):
+            return "skinny"
+        if not self.own_gemm and (out_dtype == torch.bfloat16 or self._library_fp32_out):
+            return "library"
+        return "mfma" if K % 8 == 0 else "plain"
+
+    def route_gated(self, M, I, K):
+        hit = self.product_plan.get((self._rows_step(M), I, K, True, torch.bfloat16))
+        if hit is not None:
+            return hit
+        if self.use_resident(M, I, K, True):
+            return "resident512" if M <= 8 else "resident256"
+        if 0 < M <= self.gated_skinny_rows and K % 8 == 0:
+            return "skinny"
+        return "two"
+
+    def _linear_by(self, how, x, w, out_dtype):
+        M, K = x.shape
+        N = w.shape[0]
+        if how == "library":
+            if out_dtype == torch.bfloat16:
+                return torch.matmul(x, w.t())          # library product, as the reference's F.linear
+            return torch.mm(x, w.t(), out_dtype=torch.float32)   # bf16 operands, 32-bit sums and results
+        y = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        if how.startswith("resident"):
+            self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, _code(out_dtype),
+                                                       int(how[8:]), self._stream()), "gemm_resident")
+        elif how == "skinny":
+            self._check(self.lib.ra_gemm_skinny_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
+                                                     self.skinny_max_grid, self._stream()), "gemm_skinny")
+        elif how == "mfma":
+            self._check(self.lib.ra_gemm_mfma_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
+                                                   self._stream()), "gemm_mfma")
+        else:
+            self._check(self.lib.ra_gemm_nt(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(x.dtype),
+                                            _code(out_dtype), self._stream()), "gemm_nt")
+        return y
+
     def linear(self, x, w, out_dtype=None):
         """y = x @ w^T, x [M, K], w [N, K]."""
         self._want(x, "x", dims=2)
@@ -288,31 +351,24 @@ class HipOps:
         if w.shape[1] != K:
             raise KernelError(f"linear: x {tuple(x.shape)} times weight {tuple(w.shape)}^T")
         out_dtype = out_dtype or x.dtype
-        if x.dtype == torch.bfloat16 and out_dtype in (torch.bfloat16, torch.float32) and \
-                self.use_resident(M, N, K, False):
-            y = torch.empty(M, N, dtype=out_dtype, device=self.device)
-            self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, _code(out_dtype),
-                                                       512 if M <= 8 else 256, self._stream()), "gemm_resident")
-            return y
-        if x.dtype == torch.bfloat16 and M > 0 and self.use_skinny(M, N, K, out_dtype):
-            y = torch.empty(M, N, dtype=out_dtype, device=self.device)
-            self._check(self.lib.ra_gemm_skinny_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
-                                                     self.skinny_max_grid, self._stream()), "gemm_skinny")
-            return y
-        if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and M > 0 and not self.own_gemm:
-            return torch.matmul(x, w.t())          # library product, as the reference's F.linear
-        if x.dtype == torch.bfloat16 and out_dtype == torch.float32 and M > 0 and not self.own_gemm \
-                and self._library_fp32_out:
-            return torch.mm(x, w.t(), out_dtype=torch.float32)   # bf16 operands, 32-bit sums and results
-        if x.dtype == torch.bfloat16 and M > 0 and K % 8 == 0:
-            y = torch.empty(M, N, dtype=out_dtype, device=self.device)
-            self._check(self.lib.ra_gemm_mfma_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(out_dtype),
-                                                   self._stream()), "gemm_mfma")
-            return y
-        y = torch.empty(M, N, dtype=out_dtype, device=self.device)
-        self._check(self.lib.ra_gemm_nt(_ptr(x), _ptr(w), _ptr(y), M, N, K, _code(x.dtype),
-                                        _code(out_dtype), self._stream()), "gemm_nt")
-        return y
+        if M == 0 or x.dtype != torch.bfloat16:
+            return self._linear_by("plain", x, w, out_dtype)      # float32: true 32-bit FMA products
+        return self._linear_by(self.route_linear(M, N, K, out_dtype), x, w, out_dtype)
+
+    def _gated_by(self, how, x, w_gate_up):
+        M, K = x.shape
+        I = w_gate_up.shape[0] // 2
+        out = torch.empty(M, I, dtype=x.dtype, device=self.device)
+        if how.startswith("resident"):
+            self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K, 1,
+                                                       _code(x.dtype), int(how[8:]), self._stream()),
+                        "gemm_resident_gated")
+        elif how == "skinny":
+            self._check(self.lib.ra_gemm_skinny_gated_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K,
+                                                           self._stream()), "gemm_skinny_gated")
+        else:
+            self.silu_mul(self.linear(x, w_gate_up), out)
+        return out
 
     def linear_silu_mul(self, x, w_gate_up):
         """silu(x @ Wg^T) * (x @ Wu^T) for w_gate_up = [Wg; Wu]: one kernel for few rows, else two."""
@@ -322,18 +378,83 @@ class HipOps:
         I = w_gate_up.shape[0] // 2
         if w_gate_up.shape[1] != K or w_gate_up.shape[0] != 2 * I:
             raise KernelError(f"linear_silu_mul: x {tuple(x.shape)}, weight {tuple(w_gate_up.shape)}")
-        out = torch.empty(M, I, dtype=x.dtype, device=self.device)
-        if x.dtype == torch.bfloat16 and self.use_resident(M, I, K, True):
-            self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K, 1,
-                                                       _code(x.dtype), 512 if M <= 8 else 256, self._stream()),
-                        "gemm_resident_gated")
-            return out
-        if x.dtype == torch.bfloat16 and 0 < M <= self.gated_skinny_rows and K % 8 == 0:
-            self._check(self.lib.ra_gemm_skinny_gated_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K,
-                                                           self._stream()), "gemm_skinny_gated")
-            return out
-        self.silu_mul(self.linear(x, w_gate_up), out)
-        return out
+        how = self.route_gated(M, I, K) if x.dtype == torch.bfloat16 and M > 0 else "two"
+        return self._gated_by(how, x, w_gate_up)
+
+    def _candidates(self, M, N, K, gated, out_dtype):
+        """The ways that can form this product at all."""
+        if gated:
+            c = ["two"]
+            if M <= 16 and K % 8 == 0:
+                c.append("skinny")
+        else:
+            c = ["library"] if out_dtype == torch.bfloat16 or self._library_fp32_out else []
+            if M <= 64 and K % 8 == 0:
+                c.append("skinny")
+        if self.lib.ra_gemm_resident_fits(M, K, 1 if gated else 0):
+            c += ["resident256", "resident512"]
+        return c
+
+    def tune_products(self, products, max_rows=64, margin=0.93):
+        """Measures, for every shape among ``products`` and every row count of ROW_STEPS up to max_rows,
+        the ways to form the product, and notes the fastest in product_plan where it beats the rule's
+        choice by more than the margin (so that noise does not move a choice to and fro).
+
+        products: (weight [N, K] bfloat16, gated, out_dtype) of the model's projections. The weights
+        of one shape are taken in turn, as a decode step reads them: from memory, not from a cache
+        that a repeated product on one weight would sit in. A few milliseconds per shape and row count."""
+        groups = {}
+        for w, gated, out_dtype in products:
+            if w.dtype != torch.bfloat16 or w.dim() != 2 or w.device != self.device:
+                continue
+            N = w.shape[0] // 2 if gated else w.shape[0]
+            groups.setdefault((N, w.shape[1], bool(gated), out_dtype or torch.bfloat16), []).append(w)
+        for (N, K, gated, out_dtype), ws in groups.items():
+            seen, uniq = set(), []
+            for w in ws:                                  # tied weights are listed once
+                if w.data_ptr() not in seen:
+                    seen.add(w.data_ptr())
+                    uniq.append(w)
+            launches = max(4, min(16, len(uniq)))
+            for rows in self.ROW_STEPS:
+                if rows > max(1, max_rows) and rows != self._rows_step(max_rows):
+                    continue
+                key = (rows, N, K, gated, out_dtype)
+                if key in self.product_plan or key in self._tuned:
+                    continue
+                self._tuned.add(key)
+                cands = self._candidates(rows, N, K, gated, out_dtype)
+                rule = self.route_gated(rows, N, K) if gated else self.route_linear(rows, N, K, out_dtype)
+                if len(cands) < 2 or rule not in cands:
+                    continue
+                x = torch.randn(rows, K, device=self.device, dtype=torch.float32).to(torch.bfloat16)
+                times = {}
+                for how in cands:
+                    run = (lambda w, how=how: self._gated_by(how, x, w)) if gated else \
+                          (lambda w, how=how: self._linear_by(how, x, w, out_dtype))
+                    times[how] = self._time_over(run, uniq, launches)
+                best = min(times, key=times.get)
+                if best != rule and times[best] < margin * times[rule]:
+                    self.product_plan[key] = best
+
+    def _time_over(self, run, weights, launches):
+        """Seconds per call of run(w), the weights taken in turn, launched from one captured graph."""
+        import time
+        run(weights[0])
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(launches):
+                run(weights[i % len(weights)])
+        graph.replay()
+        torch.cuda.synchronize(self.device)
+        best = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize(self.device)
+            best = min(best, time.perf_counter() - t0)
+        return best / launches
 
     # ------------------------------------------------------------------ attention
     def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):

@@ -43,7 +43,7 @@ class LinearHead:
 
     def __init__(self, params, tensors, rt, shared=None):
         self.rt = rt
-        self.weight = rt.matrix(tensors["weight"])
+        self.weight = rt.product(rt.matrix(tensors["weight"]), out_dtype=torch.float32)
 
     def forward(self, x):
         return self.rt.ops.linear(x, self.weight, out_dtype=torch.float32)

@@ -23,9 +23,9 @@ class SwiGLU:
     def __init__(self, params, tensors, rt, shared=None):
         self.rt = rt
         self.inter = int(params["intermediate_size"])
-        self.w_gate_up = torch.cat([rt.matrix(tensors["gate_proj"]), rt.matrix(tensors["up_proj"])],
-                                   dim=0).contiguous()
-        self.w_down = rt.matrix(tensors["down_proj"])
+        self.w_gate_up = rt.product(torch.cat([rt.matrix(tensors["gate_proj"]), rt.matrix(tensors["up_proj"])],
+                                              dim=0).contiguous(), gated=True)
+        self.w_down = rt.product(rt.matrix(tensors["down_proj"]))
 
     def forward(self, x, step=None):
         ops = self.rt.ops

@@ -28,6 +28,7 @@ class Runtime:
             ops = HipOps(self.device)
         self.ops = ops
         self._cast: Dict[int, torch.Tensor] = {}
+        self.products = []                  # (weight, gated, result dtype) of the parts' matrix products
 
     # ---- weight preparation -------------------------------------------------
     def matrix(self, t: torch.Tensor) -> torch.Tensor:
@@ -42,6 +43,13 @@ class Runtime:
             hit = (t, t.to(device=self.device, dtype=self.dtype).contiguous())
             self._cast[key] = hit
         return hit[1]
+
+    def product(self, w: torch.Tensor, gated: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """Notes that the part will multiply by w (ops.linear, or ops.linear_silu_mul when gated) and
+        returns w. The kernel set may measure, once the model is built, which of its ways to form the
+        products of these shapes is fastest; a part that does not note its weights is served by rules."""
+        self.products.append((w, gated, out_dtype))
+        return w
 
     def vector32(self, t: torch.Tensor) -> torch.Tensor:
         """A small vector (norm weight) as 32-bit floats; bf16 values convert exactly."""

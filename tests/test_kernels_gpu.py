@@ -220,6 +220,76 @@ def test_resident_product(ops, ref, M, N, K, grid):
     assert not ops.lib.ra_gemm_resident_fits(16, 8192, 0) and ops.lib.ra_gemm_resident_fits(8, 8192, 0)
 
 
+@pytest.mark.parametrize("N,K", [(331, 120), (1000, 264), (48, 4096)])
+def test_every_way_to_form_a_product(ops, monkeypatch, N, K):
+    """linear and linear_silu_mul under every way the plan may name, at every measured row count:
+    whatever the measurement at load time picks, the product is the product."""
+    plan = {}
+    monkeypatch.setattr(ops, "product_plan", plan)
+    w = rnd(2 * N, K, dtype=torch.bfloat16, seed=4, scale=0.2)
+    ways = set()
+    for M in (1, 3, 8, 11, 16, 33, 64):
+        x = rnd(M, K, dtype=torch.bfloat16, seed=M)
+        want = x.double() @ w.double().t()
+        for out_dtype in (torch.bfloat16, torch.float32):
+            for how in ops._candidates(M, 2 * N, K, False, out_dtype):
+                plan.clear()
+                plan[(ops._rows_step(M), 2 * N, K, False, out_dtype)] = how
+                assert ops.route_linear(M, 2 * N, K, out_dtype) == how
+                y = ops.linear(x, w, out_dtype=out_dtype)
+                assert y.dtype == out_dtype
+                if out_dtype == torch.float32:
+                    torch.testing.assert_close(y.double(), want, atol=1e-4 * K ** 0.5, rtol=1e-5)
+                else:
+                    torch.testing.assert_close(y.float(), want.float(), **tol(torch.bfloat16))
+                ways.add(how)
+        g, u = want[:, :N], want[:, N:]
+        for how in ops._candidates(M, N, K, True, torch.bfloat16):
+            plan.clear()
+            plan[(ops._rows_step(M), N, K, True, torch.bfloat16)] = how
+            y = ops.linear_silu_mul(x, w)
+            torch.testing.assert_close(y.float(), (g * torch.sigmoid(g) * u).float(), **tol(torch.bfloat16))
+            ways.add("gated " + how)
+    assert {"library", "skinny", "resident256", "resident512", "gated two", "gated skinny", "gated resident512"} <= ways
+
+
+def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
+    """tune_products measures every shape at every row count up to the limit, once, and notes only
+    ways that exist; a measured choice is what route_* returns from then on."""
+    from return_amd.kernels import hip_ops
+    plan, measured = {}, set()
+    monkeypatch.setattr(ops, "product_plan", plan)
+    monkeypatch.setattr(ops, "_tuned", measured)
+    ws = [rnd(768, 256, dtype=torch.bfloat16, seed=i, scale=0.1) for i in range(3)]
+    head = rnd(1000, 256, dtype=torch.bfloat16, seed=9, scale=0.1)
+    products = [(w, True, None) for w in ws] + [(w, False, None) for w in ws] + [(head, False, torch.float32)]
+    ops.tune_products(products, max_rows=5)
+    steps = [r for r in ops.ROW_STEPS if r <= 8]                     # 5 rows are served by the step of 8
+    assert measured == {(r, 384, 256, True, torch.bfloat16) for r in steps} | \
+        {(r, 768, 256, False, torch.bfloat16) for r in steps} | {(r, 1000, 256, False, torch.float32) for r in steps}
+    for (rows, N, K, gated, out_dtype), how in plan.items():
+        assert how in ops._candidates(rows, N, K, gated, out_dtype)
+        assert (ops.route_gated(rows, N, K) if gated else ops.route_linear(rows, N, K, out_dtype)) == how
+    before = dict(plan)
+    calls = []
+    monkeypatch.setattr(ops, "_time_over", lambda *a: calls.append(a) or 1.0)
+    ops.tune_products(products, max_rows=5)                            # nothing is measured twice
+    assert not calls and plan == before
+    # a way that is clearly faster replaces the rule's, one that is barely faster does not
+    cands = ops._candidates(1, 768, 256, False, torch.bfloat16)
+    assert cands == ["library", "skinny", "resident256", "resident512"]
+    plan.clear()
+    assert ops.route_linear(1, 768, 256, torch.bfloat16) == "skinny"            # the rule
+    key = (1, 768, 256, False, torch.bfloat16)
+    for seconds, choice in (([1.0, 0.95, 0.5, 0.96], "resident256"), ([0.9, 0.95, 1.0, 0.96], None)):
+        it = iter(seconds)
+        monkeypatch.setattr(ops, "_time_over", lambda *a: next(it))
+        plan.clear(); measured.clear()
+        ops.tune_products([(ws[0], False, None)], max_rows=1)
+        assert plan.get(key) == choice
+    assert hip_ops._PRODUCT_PLAN is not plan and not hip_ops._PRODUCT_PLAN.keys() & {key}
+
+
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(65, 331, 120), (128, 128, 32), (129, 257, 264), (300, 1000, 512), (70, 48, 8)])
 def test_tiled_mfma_product(ops, out_dtype, M, N, K):
