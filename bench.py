@@ -161,6 +161,7 @@ def continuous_4b(args):
     from return_amd.engine import Engine
     n = args.batch if args.batch != 8 else 128
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_4B, use_graphs=not args.no_graphs,
+                               tune_products=not args.no_tune,
                                max_token=n * 4608, max_step_tokens=512 + n, prefill_chunk=512)
     eng = Engine(runner=runner)
     rnd = random.Random(0)
@@ -198,6 +199,7 @@ def long_32b(args):
     elt = 2 if args.dtype == "bfloat16" else 4
     n, ctx, new, long_ctx = 16, 8192, max(2, args.steps), 32768
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_32B, std=0.01, use_graphs=not args.no_graphs,
+                               tune_products=not args.no_tune,
                                max_token=n * (ctx + 512) + long_ctx, max_step_tokens=ctx, prefill_chunk=ctx)
     eng = Engine(runner=runner)
     rnd = random.Random(1)
@@ -259,6 +261,9 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel from the host instead of replaying HIP graphs")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="choose the kernel of every projection by rule instead of measuring at load "
+                         "(keeps the measuring launches out of a profile)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -273,7 +278,7 @@ def main():
         return 0
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),
-                               use_graphs=not args.no_graphs)
+                               use_graphs=not args.no_graphs, tune_products=not args.no_tune)
     V = cfg.vocab_size
 
     # ---- headline: decode at the given batch
@@ -323,7 +328,7 @@ def main():
                    "intermediate": cfg.intermediate_size, "vocab": V, "global_batch": args.batch,
                    "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": PAGE,
                    "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs, "tuned_products": True,
+                   "hip_graphs": not args.no_graphs, "tuned_products": not args.no_tune,
                    "weights": "random N(0,0.02)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
