@@ -90,14 +90,36 @@ def test_trace_run_program(folder_a, tmp_path, dtype):
     compare(got, want, reqs, dtype)
 
 
-def test_long_decoding(folder_b):
-    """300 tokens one by one after a short prompt, in 32-bit."""
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folder_b, dtype):
+    """300 tokens one by one after a short prompt."""
     toks = tt.random_tokens(TINY_B["vocab_size"], 320, seed=77)
     reqs = {"long": toks}
     want = oracle(folder_b, reqs)
     steps = tt.tail_decoded(reqs, tail=300)
-    runner = make_runner(folder_b, "float32", 320)
-    compare(tt.run_in_process(runner, steps), want, reqs, "float32")
+    runner = make_runner(folder_b, dtype, 320)
+    compare(tt.run_in_process(runner, steps), want, reqs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["a", "b"])
+def test_first_tokens_of_a_sequence(folder_a, folder_b, which, dtype):
+    """The first places of a sequence, where attention has one key, then two, and the first page
+    is not yet full: one request decoded from its very first token, one that starts with two
+    tokens and goes on one by one, one that starts with three; all live together."""
+    folder, raw = (folder_a, TINY_A) if which == "a" else (folder_b, TINY_B)
+    reqs = {rid: tt.random_tokens(raw["vocab_size"], 40, seed=ord(rid)) for rid in "xyz"}
+    want = oracle(folder, reqs)
+    first = {"x": 1, "y": 2, "z": 3}
+    steps = [{"step": 0, "end": [], "entries": [
+        {"id": rid, "tokens": reqs[rid][:k], "want": list(range(k))} for rid, k in first.items()]}]
+    for i in range(1, 40):
+        entries = [{"id": rid, "tokens": [reqs[rid][k + i - 1]], "want": [0]}
+                   for rid, k in first.items() if k + i - 1 < 40]
+        steps.append({"step": i, "entries": entries, "end": [e["id"] for e in entries if first[e["id"]] + i == 40]})
+    runner = make_runner(folder, dtype, tt.peak_tokens(steps))
+    compare(tt.run_in_process(runner, steps), want, reqs, dtype)
+    assert not runner.cache.live
 
 
 ODD = [
