@@ -80,9 +80,9 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
-# One plan per process: every engine in it forms a product of a given shape the same way.
-_PRODUCT_PLAN = {}
-_PRODUCTS_MEASURED = set()
+# What tune_products has measured in this process: (row step, N, K, gated, result dtype) -> the way that
+# beat the rule's, or None where the rule stands. Every kernel set that tunes gets the same answers.
+_PRODUCTS_MEASURED = {}
 
 
 class HipOps:
@@ -106,8 +106,16 @@ class HipOps:
             self._library_fp32_out = torch.mm(a, a.t(), out_dtype=torch.float32).dtype == torch.float32
         except (TypeError, RuntimeError):
             self._library_fp32_out = False
-        self.product_plan = _PRODUCT_PLAN    # (row step, N, K, gated, result dtype) -> way, where measured faster than the rule
-        self._tuned = _PRODUCTS_MEASURED
+        # whether the library's float32 product is a true 32-bit one (against a 64-bit product; operands
+        # rounded to a shorter mantissa would be off by 1e-3)
+        g = torch.Generator(device="cpu").manual_seed(0)
+        a = torch.randn(32, 512, generator=g).to(self.device)
+        b = torch.randn(48, 512, generator=g).to(self.device)
+        want = a.double() @ b.double().t()
+        self._library_fp32_exact = bool(((torch.matmul(a, b.t()).double() - want).abs().max()
+                                         <= 2e-5 * want.abs().max()).item())
+        self.product_plan = {}               # (row step, N, K, gated, result dtype) -> way, where measured faster than the rule
+        self._measured = _PRODUCTS_MEASURED
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -351,8 +359,11 @@ class HipOps:
         if w.shape[1] != K:
             raise KernelError(f"linear: x {tuple(x.shape)} times weight {tuple(w.shape)}^T")
         out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.float32 and out_dtype == torch.float32 and M > 16 and self._library_fp32_exact \
+                and not self.own_gemm:
+            return torch.matmul(x, w.t())          # the library's float32 product: checked above to be 32-bit
         if M == 0 or x.dtype != torch.bfloat16:
-            return self._linear_by("plain", x, w, out_dtype)      # float32: true 32-bit FMA products
+            return self._linear_by("plain", x, w, out_dtype)      # float32: 32-bit FMA products, W streamed once
         return self._linear_by(self.route_linear(M, N, K, out_dtype), x, w, out_dtype)
 
     def _gated_by(self, how, x, w_gate_up):
@@ -420,22 +431,30 @@ class HipOps:
                 if rows > max(1, max_rows) and rows != self._rows_step(max_rows):
                     continue
                 key = (rows, N, K, gated, out_dtype)
-                if key in self.product_plan or key in self._tuned:
-                    continue
-                self._tuned.add(key)
-                cands = self._candidates(rows, N, K, gated, out_dtype)
-                rule = self.route_gated(rows, N, K) if gated else self.route_linear(rows, N, K, out_dtype)
-                if len(cands) < 2 or rule not in cands:
-                    continue
-                x = torch.randn(rows, K, device=self.device, dtype=torch.float32).to(torch.bfloat16)
-                times = {}
-                for how in cands:
-                    run = (lambda w, how=how: self._gated_by(how, x, w)) if gated else \
-                          (lambda w, how=how: self._linear_by(how, x, w, out_dtype))
-                    times[how] = self._time_over(run, uniq, launches)
-                best = min(times, key=times.get)
-                if best != rule and times[best] < margin * times[rule]:
-                    self.product_plan[key] = best
+                if key not in self._measured:
+                    self._measured[key] = self._measure(key, uniq, launches, margin)
+                if self._measured[key] is not None:
+                    self.product_plan[key] = self._measured[key]
+
+    def _measure(self, key, weights, launches, margin):
+        """The way that forms this product clearly faster than the rule's, or None."""
+        rows, N, K, gated, out_dtype = key
+        cands = self._candidates(rows, N, K, gated, out_dtype)
+        saved, self.product_plan = self.product_plan, {}          # the rule's choice, and "two" by the rule's product
+        try:
+            rule = self.route_gated(rows, N, K) if gated else self.route_linear(rows, N, K, out_dtype)
+            if len(cands) < 2 or rule not in cands:
+                return None
+            x = torch.randn(rows, K, device=self.device, dtype=torch.float32).to(torch.bfloat16)
+            times = {}
+            for how in cands:
+                run = (lambda w, how=how: self._gated_by(how, x, w)) if gated else \
+                      (lambda w, how=how: self._linear_by(how, x, w, out_dtype))
+                times[how] = self._time_over(run, weights, launches)
+        finally:
+            self.product_plan = saved
+        best = min(times, key=times.get)
+        return best if best != rule and times[best] < margin * times[rule] else None
 
     def _time_over(self, run, weights, launches):
         """Seconds per call of run(w), the weights taken in turn, launched from one captured graph."""

@@ -162,16 +162,18 @@ def test_silu_mul(ops, ref, dtype, T, I):
 @pytest.mark.parametrize("dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
                                              (torch.bfloat16, torch.float32)])
 @pytest.mark.parametrize("M,N,K", [(1, 331, 120), (7, 100, 77), (64, 64, 64), (65, 129, 250), (200, 48, 1000)])
-def test_linear(ops, dtype, out_dtype, M, N, K):
+def test_linear(ops, monkeypatch, dtype, out_dtype, M, N, K):
     x = rnd(M, K, dtype=dtype, seed=41)
     w = rnd(N, K, dtype=dtype, seed=42, scale=0.1)
-    y = ops.linear(x, w, out_dtype=out_dtype)
     want = x.double() @ w.double().t()
-    assert y.dtype == out_dtype and tuple(y.shape) == (M, N)
-    if out_dtype == torch.float32:
-        torch.testing.assert_close(y.double(), want, atol=2e-5 * K ** 0.5, rtol=1e-5)
-    else:
-        torch.testing.assert_close(y.double(), want, atol=3e-2, rtol=2e-2)
+    for own in (False, True):               # the library's product where it is used, and the hand-written one
+        monkeypatch.setattr(ops, "own_gemm", own)
+        y = ops.linear(x, w, out_dtype=out_dtype)
+        assert y.dtype == out_dtype and tuple(y.shape) == (M, N)
+        if out_dtype == torch.float32:
+            torch.testing.assert_close(y.double(), want, atol=2e-5 * K ** 0.5, rtol=1e-5)
+        else:
+            torch.testing.assert_close(y.double(), want, atol=3e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -254,25 +256,28 @@ def test_every_way_to_form_a_product(ops, monkeypatch, N, K):
 
 
 def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
-    """tune_products measures every shape at every row count up to the limit, once, and notes only
-    ways that exist; a measured choice is what route_* returns from then on."""
-    from return_amd.kernels import hip_ops
-    plan, measured = {}, set()
+    """tune_products measures every shape at every row count up to the limit, once in a process, and
+    notes only ways that exist; a measured choice is what route_* returns from then on; a kernel
+    set that has not tuned follows the rules."""
+    from return_amd.kernels.hip_ops import HipOps
+    plan, measured = {}, {}
     monkeypatch.setattr(ops, "product_plan", plan)
-    monkeypatch.setattr(ops, "_tuned", measured)
+    monkeypatch.setattr(ops, "_measured", measured)
     ws = [rnd(768, 256, dtype=torch.bfloat16, seed=i, scale=0.1) for i in range(3)]
     head = rnd(1000, 256, dtype=torch.bfloat16, seed=9, scale=0.1)
     products = [(w, True, None) for w in ws] + [(w, False, None) for w in ws] + [(head, False, torch.float32)]
     ops.tune_products(products, max_rows=5)
     steps = [r for r in ops.ROW_STEPS if r <= 8]                     # 5 rows are served by the step of 8
-    assert measured == {(r, 384, 256, True, torch.bfloat16) for r in steps} | \
+    assert set(measured) == {(r, 384, 256, True, torch.bfloat16) for r in steps} | \
         {(r, 768, 256, False, torch.bfloat16) for r in steps} | {(r, 1000, 256, False, torch.float32) for r in steps}
+    assert plan == {k: v for k, v in measured.items() if v is not None}
     for (rows, N, K, gated, out_dtype), how in plan.items():
         assert how in ops._candidates(rows, N, K, gated, out_dtype)
         assert (ops.route_gated(rows, N, K) if gated else ops.route_linear(rows, N, K, out_dtype)) == how
     before = dict(plan)
     calls = []
     monkeypatch.setattr(ops, "_time_over", lambda *a: calls.append(a) or 1.0)
+    plan.clear()
     ops.tune_products(products, max_rows=5)                            # nothing is measured twice
     assert not calls and plan == before
     # a way that is clearly faster replaces the rule's, one that is barely faster does not
@@ -286,8 +291,9 @@ def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
         monkeypatch.setattr(ops, "_time_over", lambda *a: next(it))
         plan.clear(); measured.clear()
         ops.tune_products([(ws[0], False, None)], max_rows=1)
-        assert plan.get(key) == choice
-    assert hip_ops._PRODUCT_PLAN is not plan and not hip_ops._PRODUCT_PLAN.keys() & {key}
+        assert plan.get(key) == choice and measured[key] == choice
+    other = HipOps(DEV)
+    assert other.product_plan == {} and other.route_linear(1, 768, 256, torch.bfloat16) == "skinny"
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
@@ -321,15 +327,20 @@ def test_linear_float32_few_rows(ops, M, N, K):
     torch.testing.assert_close(y.double(), x.double() @ w.double().t(), atol=2e-6 * K ** 0.5 + 1e-6, rtol=1e-5)
 
 
-def test_linear_fp32_is_true_fp32(ops):
-    """Inputs 1 + 2^-12 round to 1 in bf16 and tf32; a true 32-bit product keeps the 2^-11 per term."""
+@pytest.mark.parametrize("M,own", [(4, False), (40, False), (40, True), (300, False)])
+def test_linear_fp32_is_true_fp32(ops, monkeypatch, M, own):
+    """Inputs 1 + 2^-12 round to 1 in bf16 and tf32; a true 32-bit product keeps the 2^-11 per term.
+    Few rows (the kernel that streams W once), many rows through the library (which the kernel set
+    has checked at start to be a 32-bit product) and through the hand-written tiled kernel."""
+    assert ops._library_fp32_exact
+    monkeypatch.setattr(ops, "own_gemm", own)
     K = 64
-    x = torch.full((4, K), 1.0 + 2.0 ** -12, device=DEV)
+    x = torch.full((M, K), 1.0 + 2.0 ** -12, device=DEV)
     w = torch.full((8, K), 1.0 + 2.0 ** -12, device=DEV)
     y = ops.linear(x, w)
     want = K * (1.0 + 2.0 ** -12) ** 2          # 64.03125...
     assert abs(float(y[0, 0]) - want) < 1e-4
-    assert abs(float(y[3, 7]) - want) < 1e-4
+    assert abs(float(y[M - 1, 7]) - want) < 1e-4
 
 
 def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
