@@ -523,6 +523,25 @@ def test_attention_far_key_stands_out(ops, dtype):
     torch.testing.assert_close(out[0, ::2].float(), want, atol=3e-2, rtol=3e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_over_a_long_context(ops, ref, dtype):
+    """40,000 keys in scattered pages: a decoded token at the end of them, one after five keys, and
+    a portion of 300 query rows whose first row sees 39,700 keys; in one step."""
+    Hq, Hkv, D, P = 8, 2, 128, 16
+    segs = [(1, 39_999), (1, 5), (300, 39_700)]
+    need = [-(-(a + b) // P) for a, b in segs]
+    perm = torch.randperm(sum(need) + 7, generator=torch.Generator().manual_seed(3)).tolist()
+    pages_of = [[perm.pop() for _ in range(k)] for k in need]
+    step = _step([s[0] for s in segs], [s[1] for s in segs], P, pages_of)
+    kp = rnd(sum(need) + 7, P, Hkv, D, dtype=dtype, seed=81)
+    vp = rnd(sum(need) + 7, P, Hkv, D, dtype=dtype, seed=82)
+    q = rnd(sum(s[0] for s in segs), Hq, D, dtype=dtype, seed=83)
+    a, b = torch.zeros_like(q), torch.zeros_like(q)
+    ops.attention(q, a, kp, vp, step, 0, D ** -0.5, 0)
+    ref.attention(q, b, kp, vp, step, 0, D ** -0.5, 0)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
 @pytest.mark.parametrize("V", [331, 5000])
 def test_sample_greedy_and_logprob(ops, V):
     logits = rnd(6, V, seed=71, scale=3.0)
