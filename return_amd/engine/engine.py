@@ -64,15 +64,21 @@ class Engine:
     def submit(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
                request_id=None) -> Request:
         params = params or SamplingParams()
+        self.check_prompt(prompt_ids)
         n = self._submitted
         self._submitted += 1
         r = Request(request_id if request_id is not None else n, prompt_ids, params)
-        for t in r.prompt_ids:
-            if not 0 <= t < self.runner.vocab_size:
-                raise ValueError(f"prompt token {t} outside the vocabulary of {self.runner.vocab_size}")
         r.stream = UniformStream(self.config.seed, params.seed if params.seed is not None else n)
         self.scheduler.add(r)
         return r
+
+    def check_prompt(self, prompt_ids: Sequence[int], name="the request") -> None:
+        """Raises ValueError for a prompt that can never run: empty, or a token outside the vocabulary."""
+        if len(prompt_ids) == 0:
+            raise ValueError(f"{name} has an empty prompt")
+        for t in prompt_ids:
+            if not 0 <= int(t) < self.runner.vocab_size:
+                raise ValueError(f"{name}: prompt token {t} outside the vocabulary of {self.runner.vocab_size}")
 
     # ------------------------------------------------------------------ one step
     def _launch_decode(self, plan, previous=None):
@@ -154,6 +160,8 @@ class Engine:
             params = [params or SamplingParams()] * len(prompts)
         if len(params) != len(prompts):
             raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling parameter sets")
+        for i, p in enumerate(prompts):               # all of them before any is queued
+            self.check_prompt(p, f"prompt {i}")
         requests = [self.submit(p, sp) for p, sp in zip(prompts, params)]
         while self.scheduler.has_work() or self._in_flight is not None:
             before = (self.steps, len(self.scheduler.waiting), len(self.scheduler.running))

@@ -77,6 +77,19 @@ def test_stop_sequence_through_the_entry_point(folder_a):
     assert r.output_ids == want and len(want) < 8 and r.finish_reason == "stop"
 
 
+def test_a_bad_prompt_is_refused_before_any_is_queued(folder_a):
+    eng = Engine(runner=runner_for(folder_a, 256))
+    sp = SamplingParams(temperature=0.0, max_new_tokens=2)
+    for bad, why in (([], "empty prompt"), ([1, TINY_A["vocab_size"]], "outside the vocabulary")):
+        with pytest.raises(ValueError, match=why):
+            eng.generate([[1, 2, 3], bad, [4, 5]], sp)
+        assert not eng.scheduler.has_work() and not eng.runner.cache.live     # the good ones were not left behind
+    assert [r.num_tokens for r in eng.generate([[1, 2, 3], [4, 5]], sp)] == [2, 2]
+    # what can never fit gives an error result of its own, the others run
+    out = eng.generate([[1] * 256, [4, 5]], sp)
+    assert out[0].finish_reason == "error" and "max_position" in out[0].error and out[1].num_tokens == 2
+
+
 def test_step_checks(folder_a):
     from return_amd.engine import StepEntry
     runner = runner_for(folder_a, 64)
