@@ -60,13 +60,35 @@ def cmd_generate(args) -> int:
                     page_size=args.page_size, seed=args.seed, max_step_tokens=args.max_step_tokens,
                     prefill_chunk=args.prefill_chunk, use_graphs=not args.no_graphs,
                     tune_products=not args.no_tune)
-    results = engine.generate([p for _, p, _ in parsed], [sp for _, _, sp in parsed])
-    for (sid, _, _), r in zip(parsed, results):
-        out = {"session_id": sid, "output_ids": r.output_ids, "output_logprobs": r.output_logprobs,
-               "num_tokens": r.num_tokens, "finish_reason": r.finish_reason}
-        if r.error:
-            out["error"] = r.error
-        print(json.dumps(out), flush=True)
+    # Requests are run together until a session_id comes again: that request is a later turn of the
+    # session (the reference keeps a session's cache for its next request, rollout/engine.py:286-306,
+    # which sends the whole conversation again, 266-274). A session's cache is kept while more of
+    # its turns follow.
+    start = 0
+    while start < len(parsed):
+        end, seen = start, set()
+        while end < len(parsed) and parsed[end][0] not in seen:
+            seen.add(parsed[end][0])
+            end += 1
+        later = {sid for sid, _, _ in parsed[end:]}
+        turn = parsed[start:end]
+        results = [None] * len(turn)
+        for keep in (True, False):                 # one call for the sessions that go on, one for the others
+            idx = [i for i, (sid, _, _) in enumerate(turn) if (sid in later) == keep]
+            if idx:
+                got = engine.generate([turn[i][1] for i in idx], [turn[i][2] for i in idx],
+                                      session_ids=[turn[i][0] for i in idx], keep=keep)
+                for i, r in zip(idx, got):
+                    results[i] = r
+        for (sid, _, _), r in zip(turn, results):
+            out = {"session_id": sid, "output_ids": r.output_ids, "output_logprobs": r.output_logprobs,
+                   "num_tokens": r.num_tokens, "finish_reason": r.finish_reason}
+            if r.cached_tokens:
+                out["cached_tokens"] = r.cached_tokens
+            if r.error:
+                out["error"] = r.error
+            print(json.dumps(out), flush=True)
+        start = end
     if args.stats:
         print(json.dumps(engine.stats()), file=sys.stderr)
     return 0

@@ -28,6 +28,7 @@ class GenerationResult:
     num_tokens: int
     finish_reason: str                      # "length" | "stop" | "error"
     error: Optional[str] = None
+    cached_tokens: int = 0                  # tokens of the prompt that a kept session still held
 
 
 class Engine:
@@ -62,15 +63,24 @@ class Engine:
 
     # ------------------------------------------------------------------ requests
     def submit(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
-               request_id=None) -> Request:
+               request_id=None, keep: bool = False) -> Request:
+        """Queue a request. request_id names its session (the reference's session_id,
+        rollout/server.py:25-42); with keep, what the cache holds when it ends stays under that id,
+        and a later request with the same id whose prompt repeats those tokens and goes on computes
+        only the rest (rollout/engine.py:266-274, 286-306). release() gives a kept session back."""
         params = params or SamplingParams()
         self.check_prompt(prompt_ids)
         n = self._submitted
         self._submitted += 1
-        r = Request(request_id if request_id is not None else n, prompt_ids, params)
+        r = Request(request_id if request_id is not None else n, prompt_ids, params, keep=keep)
         r.stream = UniformStream(self.config.seed, params.seed if params.seed is not None else n)
         self.scheduler.add(r)
         return r
+
+    def release(self, request_id) -> bool:
+        """Give back what a kept session holds (the reference's /release, rollout/engine.py:276-284);
+        a session still under way is given back when it ends. Returns whether the id was known."""
+        return self.scheduler.release(request_id)
 
     def check_prompt(self, prompt_ids: Sequence[int], name="the request") -> None:
         """Raises ValueError for a prompt that can never run: empty, or a token outside the vocabulary."""
@@ -153,16 +163,21 @@ class Engine:
 
     # ------------------------------------------------------------------ whole jobs
     def generate(self, prompts: Sequence[Sequence[int]],
-                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None
-                 ) -> List[GenerationResult]:
-        """Generate for every prompt (lists of token ids); results come in the prompts' order."""
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 session_ids: Optional[Sequence] = None, keep: bool = False) -> List[GenerationResult]:
+        """Generate for every prompt (lists of token ids); results come in the prompts' order.
+        session_ids name the requests (distinct within one call); with keep their caches stay
+        for a later call that goes on with the same sessions."""
         if params is None or isinstance(params, SamplingParams):
             params = [params or SamplingParams()] * len(prompts)
         if len(params) != len(prompts):
             raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling parameter sets")
+        if session_ids is not None and (len(session_ids) != len(prompts) or len(set(session_ids)) != len(prompts)):
+            raise ValueError("session_ids must name every prompt, each differently")
         for i, p in enumerate(prompts):               # all of them before any is queued
             self.check_prompt(p, f"prompt {i}")
-        requests = [self.submit(p, sp) for p, sp in zip(prompts, params)]
+        requests = [self.submit(p, sp, request_id=None if session_ids is None else session_ids[i], keep=keep)
+                    for i, (p, sp) in enumerate(zip(prompts, params))]
         while self.scheduler.has_work() or self._in_flight is not None:
             before = (self.steps, len(self.scheduler.waiting), len(self.scheduler.running))
             self.step()
@@ -173,12 +188,13 @@ class Engine:
     @staticmethod
     def result_of(r: Request) -> GenerationResult:
         return GenerationResult(list(r.output), list(r.output_logprobs), len(r.output),
-                                r.finish_reason or "error", str(r.error) if r.error else None)
+                                r.finish_reason or "error", str(r.error) if r.error else None, r.resumed)
 
     def stats(self) -> dict:
         cache = self.runner.cache
         return {"steps": self.steps, "prefill_tokens": self.prefill_tokens,
                 "decode_tokens": self.decode_tokens, "step_seconds": self.step_seconds,
                 "running": len(self.scheduler.running), "waiting": len(self.scheduler.waiting),
+                "resident": len(self.scheduler.resident),
                 "kv_used": [g.pages.in_use() for g in cache.groups],
                 "kv_total": [g.num_pages for g in cache.groups]}

@@ -28,10 +28,13 @@ from ..sampling.params import SamplingParams, UniformStream, ends_with_stop
 class Request:
     """One generation request (the reference's Request, rollout/engine.py:13-62, without paragraphs)."""
 
-    def __init__(self, request_id, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None):
+    def __init__(self, request_id, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                 keep: bool = False):
         if len(prompt_ids) == 0:
             raise ValueError(f"request {request_id!r} has an empty prompt")
         self.id = request_id
+        self.keep = bool(keep)              # what the cache holds stays under this id when the request ends
+        self.resumed = 0                    # tokens of the prompt that were found in the cache at admission
         self.prompt_ids = [int(t) for t in prompt_ids]
         self.params = params or SamplingParams()
         self.output: List[int] = []
@@ -93,11 +96,41 @@ class Scheduler:
         self.waiting: Deque[Request] = collections.deque()
         self.running: List[Request] = []
         self._life_pages: Dict[object, List[int]] = {}     # request id -> pages of each group set aside
+        # Sessions that ended with keep: id -> the tokens their cache holds, oldest first. The
+        # reference keeps every session until it is released (rollout/engine.py:286-306 and 276-284);
+        # here a kept session is also given up, oldest first, when a waiting request needs its
+        # pages or its slot.
+        self.resident: "collections.OrderedDict[object, List[int]]" = collections.OrderedDict()
 
     # ------------------------------------------------------------------ queue
     def add(self, request: Request) -> None:
+        if any(r.id == request.id for r in self.running) or any(r.id == request.id for r in self.waiting):
+            raise ValueError(f"request {request.id!r} is already under way")
         request.status = "waiting"
         self.waiting.append(request)
+
+    def release(self, request_id) -> bool:
+        """Give back what a kept session holds; one still under way is given back when it ends.
+        Returns whether the id was known."""
+        if request_id in self.resident:
+            del self.resident[request_id]
+            self.cache.free_request(request_id)
+            return True
+        known = False
+        for r in list(self.running) + list(self.waiting):
+            if r.id == request_id:
+                r.keep = False
+                known = True
+        return known
+
+    def _give_up_oldest(self, spare) -> bool:
+        """Frees the kept session that was used longest ago, but not ``spare``."""
+        for rid in self.resident:
+            if rid != spare:
+                del self.resident[rid]
+                self.cache.free_request(rid)
+                return True
+        return False
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
@@ -126,11 +159,38 @@ class Scheduler:
                 return self._fail(r, KVCapacityError(
                     f"request needs {need} pages of cache group {g}, the pool has "
                     f"{self.cache.groups[g].num_pages}"))
-        if len(self.running) >= self.max_reside or self.cache.free_slots() < 1:
+        # A kept session goes on where it stopped if the prompt repeats what its cache holds and
+        # brings at least one token more (the reference strips the cached prefix unchecked,
+        # rollout/engine.py:266-274); otherwise what it holds is given back and it starts afresh.
+        held = self.resident.get(r.id)
+        if held is not None and not (len(held) < n_prompt and r.prompt_ids[:len(held)] == held):
+            del self.resident[r.id]
+            self.cache.free_request(r.id)
+            held = None
+        have = self.cache.held_pages(r.id) if held is not None else [0] * len(life)
+        others = [rid for rid in self.resident if rid != r.id]
+        if held is None and len(self.running) >= self.max_reside:
             return False
-        if any(need > free for need, free in zip(life, self._unclaimed())):
+        # kept sessions are given up only if that lets the request in
+        could = self._unclaimed()
+        for rid in others:
+            for g, h in enumerate(self.cache.held_pages(rid)):
+                could[g] += h
+        if any(need - h > c for need, h, c in zip(life, have, could)):
             return False
-        self.cache.add_request(r.id)
+        while True:
+            slots_ok = held is not None or (len(self.running) + len(self.resident) < self.max_reside
+                                            and self.cache.free_slots() >= 1)
+            pages_ok = all(need - h <= free for need, h, free in zip(life, have, self._unclaimed()))
+            if slots_ok and pages_ok:
+                break
+            if not self._give_up_oldest(spare=r.id):
+                return False
+        if held is not None:
+            del self.resident[r.id]
+            r.num_computed = r.resumed = len(held)
+        else:
+            self.cache.add_request(r.id)
         self._life_pages[r.id] = life
         r.status = "running"
         self.running.append(r)
@@ -215,7 +275,12 @@ class Scheduler:
         for r in done:
             self.running.remove(r)
             self._life_pages.pop(r.id, None)
-            self.cache.free_request(r.id)
+            if r.keep:
+                # what the cache holds by now: the prompt and the tokens fed back so far (the last one
+                # too, if the step after this one was launched before this one's tokens were read)
+                self.resident[r.id] = (r.prompt_ids + r.output)[:self.cache.seq_len(r.id)]
+            else:
+                self.cache.free_request(r.id)
         return done
 
     def abort(self, r: Request, error: BaseException) -> None:

@@ -179,3 +179,88 @@ def test_schedule_ahead_only_when_the_tokens_are_all_that_is_missing(folder_a):
     assert [e.request.id for e in ahead.entries] == ["a"] and ahead.entries[0].tokens == [None]
     sch.add(Request("c", [9], SamplingParams(max_new_tokens=2)))
     assert sch.schedule_ahead(plan) is None                  # somebody waits: the next step is not only decoding
+
+
+def engine_for(folder, lookahead=True, **kw):
+    ec = EngineConfig(dtype="float32", page_size=16, max_token=kw.pop("max_token", 1024), max_reside=kw.pop("max_reside", 4),
+                      max_step_tokens=64, prefill_chunk=24, device="cpu", lookahead=lookahead, **kw)
+    return Engine(runner=ModelRunner(folder, engine_config=ec, ops=TorchOps()))
+
+
+@pytest.mark.parametrize("lookahead", [False, True])
+def test_a_kept_session_goes_on_where_it_stopped(folder_a, lookahead):
+    """Two turns of two sessions: the second turn's prompt repeats the first turn and its answer and
+    goes on; only the rest is computed, and the answers are the plain implementation's on the
+    whole prompts. One session ends its first turn on a stop sequence, which with steps launched
+    ahead is found out after its last token was already fed."""
+    cfg, w = plain.read_folder(folder_a)
+    V = TINY_A["vocab_size"]
+    p1 = {"s": tt.random_tokens(V, 21, seed=1), "t": tt.random_tokens(V, 40, seed=2)}
+    free = plain.greedy_generate(cfg, w, p1["t"], 9)
+    sp = {"s": SamplingParams(temperature=0.0, max_new_tokens=6),
+          "t": SamplingParams(temperature=0.0, max_new_tokens=9, stop_ids=[free[3:5]])}
+    eng = engine_for(folder_a, lookahead)
+    out1 = dict(zip("st", eng.generate([p1["s"], p1["t"]], [sp["s"], sp["t"]], session_ids=["s", "t"], keep=True)))
+    assert out1["s"].output_ids == plain.greedy_generate(cfg, w, p1["s"], 6)
+    stopped = plain.greedy_generate(cfg, w, p1["t"], 9, stop_ids=[free[3:5]])
+    assert out1["t"].output_ids == stopped and out1["t"].finish_reason == "stop" and len(stopped) < 9
+    assert set(eng.runner.cache.live) == {"s", "t"} and eng.stats()["resident"] == 2
+    eng.runner.cache.check_invariants()
+    p2 = {k: p1[k] + out1[k].output_ids + tt.random_tokens(V, 7, seed=ord(k)) for k in "st"}
+    before = eng.prefill_tokens
+    out2 = dict(zip("st", eng.generate([p2["s"], p2["t"]], SamplingParams(temperature=0.0, max_new_tokens=5),
+                                       session_ids=["s", "t"])))
+    for k in "st":
+        assert out2[k].output_ids == plain.greedy_generate(cfg, w, p2[k], 5)
+    assert out2["s"].cached_tokens == len(p1["s"]) + 5                 # the sixth token was sampled, never fed
+    assert out2["t"].cached_tokens == len(p1["t"]) + len(stopped) - (0 if lookahead else 1)
+    assert eng.prefill_tokens - before == sum(len(p2[k]) - out2[k].cached_tokens for k in "st")
+    assert not eng.runner.cache.live and eng.stats()["resident"] == 0    # the second turn did not keep
+    assert all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+
+
+def test_kept_sessions_that_do_not_fit_or_do_not_match(folder_a):
+    cfg, w = plain.read_folder(folder_a)
+    V = TINY_A["vocab_size"]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=4)
+    prompts = {k: tt.random_tokens(V, 30, seed=10 + i) for i, k in enumerate("abc")}
+    eng = engine_for(folder_a, max_reside=2, max_token=160)            # ten pages, two slots
+    outs = {}
+    for k in "ab":
+        outs[k] = eng.generate([prompts[k]], sp, session_ids=[k], keep=True)[0]
+    assert list(eng.scheduler.resident) == ["a", "b"]
+    with pytest.raises(ValueError, match="each differently"):
+        eng.generate([prompts["a"], prompts["b"]], sp, session_ids=["a", "a"])
+    # a third session needs a slot: the one used longest ago is given up
+    outs["c"] = eng.generate([prompts["c"]], sp, session_ids=["c"], keep=True)[0]
+    assert list(eng.scheduler.resident) == ["b", "c"] and set(eng.runner.cache.live) == {"b", "c"}
+    # "a" comes back and starts afresh; "b" has to go for it, "c" goes on from its cache afterwards
+    nxt = {k: prompts[k] + outs[k].output_ids + [5, 6] for k in "abc"}
+    ra = eng.generate([nxt["a"]], sp, session_ids=["a"], keep=True)[0]
+    assert ra.cached_tokens == 0 and ra.output_ids == plain.greedy_generate(cfg, w, nxt["a"], 4)
+    assert list(eng.scheduler.resident) == ["c", "a"]
+    rc = eng.generate([nxt["c"]], sp, session_ids=["c"], keep=True)[0]
+    assert rc.cached_tokens == 33 and rc.output_ids == plain.greedy_generate(cfg, w, nxt["c"], 4)
+    # a prompt that does not repeat what the cache holds: the cache is dropped, the answer is right
+    other = tt.random_tokens(V, 35, seed=77)
+    rc = eng.generate([other], sp, session_ids=["c"], keep=True)[0]
+    assert rc.cached_tokens == 0 and rc.output_ids == plain.greedy_generate(cfg, w, other, 4)
+    # a request that needs more pages than are free pushes kept sessions out, but only if that helps
+    big = tt.random_tokens(V, 120, seed=5)
+    rb = eng.generate([big], sp)[0]
+    assert rb.output_ids == plain.greedy_generate(cfg, w, big, 4) and eng.stats()["resident"] < 2
+    eng.runner.cache.check_invariants()
+    # release: known ids give their pages back, unknown ones are reported
+    for rid in list(eng.scheduler.resident):
+        assert eng.release(rid)
+    assert not eng.release("nobody") and not eng.runner.cache.live
+    assert all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+    # released while under way: given back at the end although it asked to be kept
+    r = eng.submit(prompts["a"], sp, request_id="z", keep=True)
+    eng.step()
+    assert eng.release("z")
+    with pytest.raises(ValueError, match="already under way"):
+        eng.submit(prompts["b"], sp, request_id="z")
+    while eng.scheduler.has_work() or eng._in_flight is not None:
+        eng.step()
+    assert r.finish_reason == "length" and not eng.runner.cache.live

@@ -104,6 +104,58 @@ def test_command_line(folder_a, tmp_path):
     assert bad.returncode != 0 and "paragraph" in bad.stderr
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_kept_sessions_on_the_gpu(folder_b, dtype):
+    """Three turns of three sessions through the graphs: every turn repeats the conversation so far
+    and adds to it; only the addition is computed. In 32-bit the answers are the plain
+    implementation's on the whole prompts; in bfloat16 every token is the plain implementation's
+    choice at its place, or its second choice where the two are nearly tied."""
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    cfg, w = plain.read_folder(folder_b)
+    V = TINY_B["vocab_size"]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=7)
+    eng = Engine(folder_b, dtype=dtype, page_size=16, max_token=2048, max_reside=4, max_step_tokens=64, prefill_chunk=32)
+    convs = {k: tt.random_tokens(V, n, seed=n) for k, n in (("a", 5), ("b", 33), ("c", 70))}
+    for turn in range(3):
+        ids = list(convs)
+        out = eng.generate([convs[k] for k in ids], sp, session_ids=ids, keep=turn < 2)
+        for k, r in zip(ids, out):
+            if dtype == "float32":
+                assert r.output_ids == plain.greedy_generate(cfg, w, convs[k], 7)
+            else:
+                rows = plain.logits(cfg, w, convs[k] + r.output_ids[:-1])[len(convs[k]) - 1:]
+                for row, tok in zip(rows, r.output_ids):
+                    top = row.topk(2)
+                    assert tok == int(top.indices[0]) or \
+                        (tok == int(top.indices[1]) and float(top.values[0] - top.values[1]) < 0.05)
+            assert (r.cached_tokens > 0) == (turn > 0) and r.cached_tokens < len(convs[k])
+            convs[k] = convs[k] + r.output_ids + tt.random_tokens(V, 3 + turn, seed=turn * 10 + len(convs[k]))
+        eng.runner.cache.check_invariants()
+    assert not eng.runner.cache.live and all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+
+
+def test_command_line_turns_of_a_session(folder_a, tmp_path):
+    """A session_id that comes again is the session's next turn: its cache was kept for it."""
+    cfg, w = plain.read_folder(folder_a)
+    first = tt.random_tokens(256, 19, seed=3)
+    a1 = plain.greedy_generate(cfg, w, first, 4)
+    second = first + a1 + [7, 8, 9]
+    reqs = [{"session_id": "s", "prompt_ids": first, "max_new_tokens": 4, "temperature": 0.0},
+            {"session_id": "u", "prompt_ids": [5, 6], "max_new_tokens": 2, "temperature": 0.0},
+            {"session_id": "s", "prompt_ids": second, "max_new_tokens": 3, "temperature": 0.0}]
+    out = subprocess.run([sys.executable, "-m", "return_amd.cli", "generate", "--model", folder_a, "--dtype", "float32",
+                          "--max-reside", "4", "--max-token", "1024", "--requests", "-", "--stats"], cwd=ROOT,
+                         input="\n".join(json.dumps(r) for r in reqs), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    lines = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    assert [l["session_id"] for l in lines] == ["s", "u", "s"]
+    assert lines[0]["output_ids"] == a1 and lines[2]["output_ids"] == plain.greedy_generate(cfg, w, second, 3)
+    assert lines[2]["cached_tokens"] == len(first) + 3 and "cached_tokens" not in lines[1]
+    stats = json.loads(out.stderr.strip().splitlines()[-1])
+    assert stats["resident"] == 0 and stats["kv_used"] == [0]
+
+
 def test_the_library_is_the_one_that_runs():
     """The HIP library is loaded in this process; there is nothing else behind the kernels."""
     from return_amd.kernels.hip_ops import HipOps
