@@ -140,3 +140,60 @@ def test_sampling_params_checks():
         Request("e", [])
     p = SamplingParams()                                               # the reference's defaults, rollout/engine.py:17-21
     assert (p.temperature, p.top_p, p.top_k, p.max_new_tokens, p.stop_ids) == (1.0, 1.0, 0, 32, [])
+
+
+def test_kept_sessions_hold_pages_until_somebody_needs_them():
+    """A kept session holds its pages and slot, resumes from them, and is given up for a waiting
+    request only if that lets the request in; random turns never lose or double a page."""
+    cm, s = make(page=4, max_token=48, max_reside=3, budget=32, chunk=32)      # twelve pages, three slots
+    a = Request("a", list(range(10)), SamplingParams(max_new_tokens=3), keep=True)
+    s.add(a)
+    drive(cm, s)
+    assert list(s.resident) == ["a"] and s.resident["a"] == list(range(10)) + [7, 7]
+    assert cm.held_pages("a") == [3] and cm.free_pages() == [9]
+    # a running request that has set aside most of the pool: the waiting one cannot get in even
+    # without "a", so "a" stays
+    b = Request("b", list(range(12)), SamplingParams(max_new_tokens=12))        # 23 tokens: six pages
+    c = Request("c", list(range(20)), SamplingParams(max_new_tokens=9))         # 28 tokens: seven pages
+    s.add(b); s.add(c)
+    plan = s.schedule()
+    assert [e.request.id for e in plan.entries] == ["b"] and list(s.resident) == ["a"] and c.status == "waiting"
+    cm.begin_step([("b", 12)]); cm.end_step()
+    s.finish_step(plan, {"b": (7, -1.0)})
+    drive(cm, s)                                     # b ends, then c fits beside "a" (3 + 7 pages of 12)
+    assert c.finish_reason == "length" and list(s.resident) == ["a"]
+    # the next turn of "a": only the new tokens are planned
+    a2 = Request("a", list(range(10)) + [7, 7, 7, 1, 2], SamplingParams(max_new_tokens=2), keep=True)
+    s.add(a2)
+    plan = s.schedule()
+    assert [(e.request.id, e.tokens) for e in plan.entries] == [("a", [7, 1, 2])] and a2.resumed == 12
+    cm.begin_step([("a", 3)]); cm.end_step()
+    s.finish_step(plan, {"a": (9, -1.0)})
+    drive(cm, s, pick=lambda r: 9)
+    assert s.resident["a"] == list(range(10)) + [7, 7, 7, 1, 2, 9]
+    # a request that needs the whole pool pushes "a" out
+    d = Request("d", list(range(40)), SamplingParams(max_new_tokens=8))
+    s.add(d)
+    drive(cm, s)
+    assert d.finish_reason == "length" and not s.resident and not cm.live
+    # random turns of five sessions in three slots
+    rnd = random.Random(3)
+    convs = {k: [rnd.randrange(50) for _ in range(rnd.randint(1, 9))] for k in "vwxyz"}
+    for _ in range(60):
+        ks = rnd.sample(sorted(convs), rnd.randint(1, 4))
+        reqs = [Request(k, convs[k], SamplingParams(max_new_tokens=rnd.randint(1, 4)), keep=rnd.random() < 0.7) for k in ks]
+        for r in reqs:
+            s.add(r)
+        drive(cm, s, pick=lambda r: len(r.output) + 1)
+        for r in reqs:
+            assert r.finish_reason == "length" and r.resumed < len(r.prompt_ids)
+            convs[r.id] = (r.prompt_ids + r.output + [rnd.randrange(50)])[-30:] if rnd.random() < 0.2 else \
+                r.prompt_ids + r.output + [rnd.randrange(50)]
+            if len(convs[r.id]) > 30:
+                convs[r.id] = [rnd.randrange(50) for _ in range(rnd.randint(1, 9))]
+        assert set(cm.live) == set(s.resident) and len(s.resident) <= 3
+        if rnd.random() < 0.2 and s.resident:
+            assert s.release(rnd.choice(list(s.resident)))
+    for rid in list(s.resident):
+        s.release(rid)
+    assert not cm.live and cm.free_pages() == [12]
