@@ -59,6 +59,8 @@ class Engine:
         self.prefill_tokens = 0
         self.decode_tokens = 0
         self.step_seconds = 0.0
+        self.decode_seconds = 0.0
+        self.prefill_seconds = 0.0
         self.steps = 0
 
     # ------------------------------------------------------------------ requests
@@ -114,7 +116,12 @@ class Engine:
             else:
                 self.prefill_tokens += len(e.tokens)
         ended = self.scheduler.finish_step(plan, sampled)
-        self.step_seconds += time.perf_counter() - t0
+        dt = time.perf_counter() - t0
+        self.step_seconds += dt
+        if all(len(e.tokens) == 1 and e.sample for e in plan.entries):
+            self.decode_seconds += dt               # steps that only decode
+        else:
+            self.prefill_seconds += dt              # steps that bring prompt portions (decoded tokens beside them)
         self.steps += 1
         return ended
 
@@ -194,6 +201,10 @@ class Engine:
         cache = self.runner.cache
         return {"steps": self.steps, "prefill_tokens": self.prefill_tokens,
                 "decode_tokens": self.decode_tokens, "step_seconds": self.step_seconds,
+                # the reference's decode_tps / prefill_tps (rollout/engine.py:104-110): tokens over the
+                # time of the steps of that kind (decoded tokens of mixed steps count as decoded)
+                "decode_tps": self.decode_tokens / self.decode_seconds if self.decode_seconds > 0 else None,
+                "prefill_tps": self.prefill_tokens / self.prefill_seconds if self.prefill_seconds > 0 else None,
                 "running": len(self.scheduler.running), "waiting": len(self.scheduler.waiting),
                 "resident": len(self.scheduler.resident),
                 "kv_used": [g.pages.in_use() for g in cache.groups],
