@@ -582,3 +582,49 @@ def test_sample_distribution(ops):
     p = (logits[0].double().cpu() / 0.8).softmax(-1)
     chi2 = float(((counts - N * p) ** 2 / (N * p)).sum())
     assert chi2 < 30.0, (chi2, counts.tolist())
+
+
+def test_calls_that_do_not_fit_are_refused_before_anything_runs(ops):
+    """Shapes, dtypes, devices and layouts that a kernel does not take raise KernelError on the
+    host; sizes beyond a kernel's limits too."""
+    from return_amd.kernels.hip_ops import KernelError
+    bf, f32 = torch.bfloat16, torch.float32
+    x, w = rnd(4, 64, dtype=bf), rnd(8, 64, dtype=bf)
+    bad = [
+        ("weight of another width", lambda: ops.linear(x, rnd(8, 48, dtype=bf))),
+        ("weight of another dtype", lambda: ops.linear(x, rnd(8, 64))),
+        ("x on the host", lambda: ops.linear(x.cpu(), w)),
+        ("x not contiguous", lambda: ops.linear(rnd(64, 4, dtype=bf).t(), w)),
+        ("gate-up with an odd number of rows", lambda: ops.linear_silu_mul(x, rnd(9, 64, dtype=bf))),
+        ("embedding into bf16", lambda: ops.embed(rnd(10, 64, dtype=bf), torch.zeros(4, dtype=torch.int32, device=DEV),
+                                                  torch.zeros(4, 64, dtype=bf, device=DEV))),
+        ("ids as int64", lambda: ops.embed(rnd(10, 64, dtype=bf), torch.zeros(4, dtype=torch.int64, device=DEV),
+                                           torch.zeros(4, 64, device=DEV))),
+        ("norm weight of another size", lambda: ops.add_rmsnorm(rnd(4, 64), None, rnd(48), 1e-6, rnd(4, 64, dtype=bf))),
+        ("delta of another shape", lambda: ops.add_rmsnorm(rnd(4, 64), rnd(3, 64, dtype=bf), rnd(64), 1e-6,
+                                                           rnd(4, 64, dtype=bf))),
+        ("silu-mul widths", lambda: ops.silu_mul(rnd(4, 100, dtype=bf), rnd(4, 60, dtype=bf))),
+        ("sampling options of another length", lambda: ops.sample(
+            rnd(3, 50), torch.zeros(2, device=DEV), torch.zeros(3, dtype=torch.int32, device=DEV),
+            torch.ones(3, device=DEV), torch.zeros(3, device=DEV))),
+        ("logits in bf16", lambda: ops.sample(
+            rnd(3, 50, dtype=bf), torch.zeros(3, device=DEV), torch.zeros(3, dtype=torch.int32, device=DEV),
+            torch.ones(3, device=DEV), torch.zeros(3, device=DEV))),
+    ]
+    # attention: heads that do not divide, a head size beyond the plain kernel's, pools that do not fit
+    step = _step([1], [5], 16, [[0]])
+    for Hq, Hkv, D, why in ((3, 2, 16, "heads"), (2, 2, 528, "head size")):
+        q = rnd(1, Hq, D, dtype=bf)
+        kp = rnd(1, 16, Hkv, D, dtype=bf)
+        bad.append((f"attention: {why}", lambda q=q, kp=kp: ops.attention(q, torch.zeros_like(q), kp, kp.clone(), step, 0, 1.0, 0)))
+    q = rnd(1, 4, 32, dtype=bf)
+    bad.append(("attention: pool of another head size",
+                lambda: ops.attention(q, torch.zeros_like(q), rnd(1, 16, 2, 16, dtype=bf), rnd(1, 16, 2, 16, dtype=bf), step, 0, 1.0, 0)))
+    bad.append(("attention: output of another shape",
+                lambda: ops.attention(q, torch.zeros(2, 4, 32, dtype=bf, device=DEV), rnd(1, 16, 2, 32, dtype=bf),
+                                      rnd(1, 16, 2, 32, dtype=bf), step, 0, 1.0, 0)))
+    for name, call in bad:
+        with pytest.raises(KernelError):
+            call()
+            pytest.fail(f"{name}: was not refused")
+    torch.cuda.synchronize()
