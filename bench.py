@@ -333,6 +333,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
+    plan = getattr(runner.rt.ops, "product_plan", None)
+    if plan:            # where the measurement at load replaced the rule: rows x N x K -> way
+        line["product_plan"] = {f"{rows}x{n}x{k}{'g' if gated else ''}": how
+                                for (rows, n, k, gated, _), how in sorted(plan.items(), key=str)}
     if prefill:
         line["prefill"] = prefill
     if points:

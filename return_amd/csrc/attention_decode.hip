@@ -58,6 +58,21 @@ __device__ __forceinline__ DecodeRange decode_range(int pos_q, int start, int wi
     return r;
 }
 
+// What the kernel needs to prepare the new token's q, k and v itself (the work of the q/k/v
+// preparation kernel: per-head RMSNorm of q and k, rotation, k and v into the cache;
+// rollout/monkey_patch/qwen3.py:29-31, 40-42 and rollout/attention.py:10-25), so that a decode
+// step has one kernel less per layer. qkv == nullptr: q is ready and the cache holds the token.
+struct DecodeFused {
+    const bf16* qkv;                  // [tokens, (Hq + 2 Hkv) D]: q heads, k heads, v heads of each token
+    const float* w_q;                 // [D] norm weights; nullptr: no norm
+    const float* w_k;
+    float eps;
+    const float* cos_t;               // [positions, D/2]; nullptr: no rotation
+    const float* sin_t;
+    bf16* k_out;                      // the pools again, to write the new token's row
+    bf16* v_out;
+};
+
 #ifdef DEC_PART
 // two floats to two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
@@ -65,14 +80,100 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
-template <int D16>
+// RMSNorm over the head and rotation of one head held as MFMA operand pieces: this lane has
+// d = 32j + 8g .. +7 of it, the four lanes l, l^16, l^32, l^48 together all of it. The rotary
+// partner of d is d + D/2, which is piece j + D32/2 of the same lane. Sums and products in
+// 32-bit, one rounding to bfloat16 at the end, as in the preparation kernel.
+template <int D32, bool NORM, bool ROPE>
+__device__ __forceinline__ void prepare_head_as(bf16x8_t (&v)[D32], const float* __restrict__ w, float eps,
+                                                const float* __restrict__ cs, const float* __restrict__ sn, int g) {
+    constexpr int D = 32 * D32;
+    // everything this lane needs of the weights and the angles, asked for at once
+    float4_t wv[NORM ? D32 : 1][2], cv[ROPE ? D32 / 2 : 1][2], sv[ROPE ? D32 / 2 : 1][2];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int j = 0; j < D32; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) wv[j][h] = *reinterpret_cast<const float4_t*>(w + 32 * j + 8 * g + 4 * h);
+    }
+    if constexpr (ROPE) {
+#pragma unroll
+        for (int j = 0; j < D32 / 2; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                cv[j][h] = *reinterpret_cast<const float4_t*>(cs + 32 * j + 8 * g + 4 * h);
+                sv[j][h] = *reinterpret_cast<const float4_t*>(sn + 32 * j + 8 * g + 4 * h);
+            }
+    }
+    float rstd = 1.0f;
+    if constexpr (NORM) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < D32; ++j) {
+            const uint4_t u = __builtin_bit_cast(uint4_t, v[j]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float lo = __uint_as_float(u[i] << 16), hi = __uint_as_float(u[i] & 0xffff0000u);
+                ss += lo * lo + hi * hi;
+            }
+        }
+        ss = rows_sum(ss);
+        rstd = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    // a piece and its rotary partner at a time
+#pragma unroll
+    for (int j = 0; j < D32 / 2; ++j) {
+        const int jp = j + D32 / 2;
+        const uint4_t ua = __builtin_bit_cast(uint4_t, v[j]), ub = __builtin_bit_cast(uint4_t, v[jp]);
+        float a[8], b[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[2 * i] = __uint_as_float(ua[i] << 16);
+            a[2 * i + 1] = __uint_as_float(ua[i] & 0xffff0000u);
+            b[2 * i] = __uint_as_float(ub[i] << 16);
+            b[2 * i + 1] = __uint_as_float(ub[i] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float x1 = a[4 * h + e], x2 = b[4 * h + e];
+                if constexpr (NORM) {
+                    x1 = x1 * rstd * wv[j][h][e];
+                    x2 = x2 * rstd * wv[jp][h][e];
+                }
+                if constexpr (ROPE) {
+                    const float y1 = x1 * cv[j][h][e] - x2 * sv[j][h][e];
+                    x2 = x2 * cv[j][h][e] + x1 * sv[j][h][e];
+                    x1 = y1;
+                }
+                a[4 * h + e] = x1;
+                b[4 * h + e] = x2;
+            }
+        const uint4_t oa = {pack2(a[0], a[1]), pack2(a[2], a[3]), pack2(a[4], a[5]), pack2(a[6], a[7])};
+        const uint4_t ob = {pack2(b[0], b[1]), pack2(b[2], b[3]), pack2(b[4], b[5]), pack2(b[6], b[7])};
+        v[j] = __builtin_bit_cast(bf16x8_t, oa);
+        v[jp] = __builtin_bit_cast(bf16x8_t, ob);
+    }
+}
+
+// w == nullptr: no norm; cs == nullptr: no rotation (the same in every lane)
+template <int D32>
+__device__ __forceinline__ void prepare_head(bf16x8_t (&v)[D32], const float* __restrict__ w, float eps,
+                                             const float* __restrict__ cs, const float* __restrict__ sn, int g) {
+    if (w != nullptr && cs != nullptr) prepare_head_as<D32, true, true>(v, w, eps, cs, sn, g);
+    else if (w != nullptr) prepare_head_as<D32, true, false>(v, w, eps, cs, sn, g);
+    else if (cs != nullptr) prepare_head_as<D32, false, true>(v, w, eps, cs, sn, g);
+}
+
+template <int D16, bool FUSED>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2 : 1))) void attn_decode_kernel(
     const bf16* __restrict__ q, float* __restrict__ part_acc, float* __restrict__ part_ml,
-    const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+    const bf16* k_pool, const bf16* v_pool,
     const int* __restrict__ page_table, const int* __restrict__ cu_pages,
     const int* __restrict__ kv_start, const int* __restrict__ cu_q,
     const int* __restrict__ q_start, const int* __restrict__ seg_ids, int Hq, int Hkv, int P,
-    float scale, int window, int split_tokens, int max_splits) {
+    float scale, int window, int split_tokens, int max_splits, DecodeFused fz) {
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;                 // full MFMA x32 steps
     constexpr bool TAIL16 = (D % 32) != 0;      // one more step, upper k half zero
@@ -101,7 +202,61 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
     const bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8_t bq[D32 > 0 ? D32 : 1];
     bf16x8_t bq_tail = z8;
-    {
+    // FUSED: the new token is not among the keys of the passes; its key and value come from the
+    // projection and are added at the end
+    [[maybe_unused]] const bool has_new = FUSED && rg.hi == pos_q;
+    const int key_hi = has_new ? pos_q - 1 : rg.hi;          // last key position read from the cache
+    const int c_begin = (rg.lo / DEC_CHUNK) * DEC_CHUNK;
+    // row in the pools of this lane's key of the pass that starts at c (clamped into the split so
+    // that every address is valid); the next pass's rows are looked up while this one's loads run
+    auto row_of = [&](int c) {
+        const int kpos = max(min(max(c + lane, rg.lo), key_hi), start);
+        const int idx = kpos - start;
+        const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
+        return pt[pi] * P + (idx - pi * P);
+    };
+    int row_next = 0;
+    [[maybe_unused]] __shared__ __attribute__((aligned(16))) uint16_t new_s[FUSED ? 2 * D : 8];   // the new token's k, v
+    if constexpr (FUSED) {
+        static_assert(!TAIL16 && D32 % 2 == 0, "the fused preparation needs a head size that is a multiple of 64");
+        const size_t width = (size_t)(Hq + 2 * Hkv) * D;
+        const bf16* tok = fz.qkv + (size_t)t * width;
+        const float* cs = fz.cos_t ? fz.cos_t + (size_t)pos_q * (D / 2) : nullptr;
+        const float* sn = fz.cos_t ? fz.sin_t + (size_t)pos_q * (D / 2) : nullptr;
+        const bf16* qp = tok + (size_t)(h0 + (n < G ? n : 0)) * D;
+#pragma unroll
+        for (int j = 0; j < D32; ++j) bq[j] = *reinterpret_cast<const bf16x8_t*>(qp + 32 * j + 8 * g);
+        row_next = row_of(c_begin);                         // asked for together with q, the weights and the angles
+        prepare_head<D32>(bq, fz.w_q, fz.eps, cs, sn, g);
+#pragma unroll
+        for (int j = 0; j < D32; ++j) bq[j] = (n < G) ? bq[j] : z8;
+        if (has_new) {
+            // The new token's key (normed, rotated) and value go into the cache for the steps to
+            // come, and into LDS for the end of this kernel. When more than 16 heads share the kv
+            // head, each of their waves writes the same bits.
+            const int idx = pos_q - start;
+            const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
+            const size_t row_new = (size_t)pt[pi] * P + (idx - pi * P);
+            bf16x8_t kn[D32];
+            const bf16* kp = tok + (size_t)(Hq + kvh) * D;
+#pragma unroll
+            for (int j = 0; j < D32; ++j) kn[j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
+            uint4_t vn = {0u, 0u, 0u, 0u};
+            if (lane < LPR) vn = *reinterpret_cast<const uint4_t*>(tok + (size_t)(Hq + Hkv + kvh) * D + lane * 8);
+            prepare_head<D32>(kn, fz.w_k, fz.eps, cs, sn, g);
+            if (n == 0) {                                   // one lane of each g holds every piece once
+#pragma unroll
+                for (int j = 0; j < D32; ++j) {
+                    *reinterpret_cast<bf16x8_t*>(fz.k_out + (row_new * Hkv + kvh) * D + 32 * j + 8 * g) = kn[j];
+                    *reinterpret_cast<bf16x8_t*>(&new_s[32 * j + 8 * g]) = kn[j];
+                }
+            }
+            if (lane < LPR) {
+                *reinterpret_cast<uint4_t*>(fz.v_out + (row_new * Hkv + kvh) * D + lane * 8) = vn;
+                *reinterpret_cast<uint4_t*>(&new_s[D + lane * 8]) = vn;
+            }
+        }
+    } else {
         const bf16* qp = q + ((size_t)t * Hq + h0 + (n < G ? n : 0)) * D;
 #pragma unroll
         for (int j = 0; j < D32; ++j) {
@@ -111,6 +266,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
         if constexpr (TAIL16) {
             if (n < G && g < 2) bq_tail = *reinterpret_cast<const bf16x8_t*>(qp + (D - 16) + 8 * g);
         }
+        row_next = row_of(c_begin);
     }
 
     const float scale2 = scale * 1.44269504088896340736f;      // scores in the base-2 domain
@@ -119,13 +275,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
 #pragma unroll
     for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int c_begin = (rg.lo / DEC_CHUNK) * DEC_CHUNK;
-    for (int c0 = c_begin; c0 <= rg.hi; c0 += DEC_CHUNK) {
-        // row of this lane's key (clamped into the split so that every address is valid)
-        const int kpos = min(max(c0 + lane, rg.lo), rg.hi);
-        const int idx = kpos - start;
-        const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
-        const int row = pt[pi] * P + (idx - pi * P);
+    for (int c0 = c_begin; c0 <= key_hi && rg.lo <= key_hi; c0 += DEC_CHUNK) {
+        const int row = row_next;
+        if (c0 + DEC_CHUNK <= key_hi) row_next = row_of(c0 + DEC_CHUNK);
 
         // ---- K tiles straight into MFMA A operands
         bf16x8_t ak[4][D32 > 0 ? D32 : 1];
@@ -177,7 +329,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int kp_abs = c0 + st * 16 + 4 * g + i;
-                const bool ok = kp_abs >= rg.lo && kp_abs <= rg.hi;
+                const bool ok = kp_abs >= rg.lo && kp_abs <= key_hi;
                 s[st][i] = ok ? cs[st][i] * scale2 : -INFINITY;
                 mx = fmaxf(mx, s[st][i]);
             }
@@ -226,6 +378,41 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
     }
     MFMA_SETTLE();
 
+    if constexpr (FUSED) {
+        if (has_new) {
+            // ---- the new token as one more key: its score by plain 32-bit sums of bf16 products
+            // (this lane's 8*D32 elements, then over the four lanes of the head), then the same
+            // running maximum and sums as in a pass
+            __syncthreads();
+            float dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < D32; ++j) {
+                const uint4_t kq = __builtin_bit_cast(uint4_t, bq[j]);
+                const uint4_t kk = *reinterpret_cast<const uint4_t*>(&new_s[32 * j + 8 * g]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    dot = fmaf(__uint_as_float(kq[i] << 16), __uint_as_float(kk[i] << 16), dot);
+                    dot = fmaf(__uint_as_float(kq[i] & 0xffff0000u), __uint_as_float(kk[i] & 0xffff0000u), dot);
+                }
+            }
+            const float sc = rows_sum(dot) * scale2;
+            const float m_new = fmaxf(m_run, sc);
+            const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+            const float pr = __builtin_amdgcn_exp2f(sc - m_new);
+            l_run = l_run * alpha + pr;
+            m_run = m_new;
+#pragma unroll
+            for (int dt = 0; dt < D16; ++dt) {
+                const uint32_t* vp2 = reinterpret_cast<const uint32_t*>(&new_s[D + dt * 16 + 4 * g]);
+                const uint32_t v01 = vp2[0], v23 = vp2[1];
+                acc[dt][0] = fmaf(pr, __uint_as_float(v01 << 16), acc[dt][0] * alpha);
+                acc[dt][1] = fmaf(pr, __uint_as_float(v01 & 0xffff0000u), acc[dt][1] * alpha);
+                acc[dt][2] = fmaf(pr, __uint_as_float(v23 << 16), acc[dt][2] * alpha);
+                acc[dt][3] = fmaf(pr, __uint_as_float(v23 & 0xffff0000u), acc[dt][3] * alpha);
+            }
+        }
+    }
+
     // ---- partial results of this split: lane (n, g) holds head n, columns 16dt + 4g .. +3
     if (n < G) {
         float* pa = part_acc + (((size_t)di * Hq + h0 + n) * max_splits + sp) * D;
@@ -247,11 +434,17 @@ extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t s
                                               const int* cup, const int* kvs, const int* cuq,
                                               const int* qs, const int* segs, int Hq, int Hkv, int P,
                                               float scale, int window, int split_tokens,
-                                              int max_splits) {
+                                              int max_splits, DecodeFused fz) {
+    if (fz.qkv != nullptr) {                      // head sizes 64, 128, 192, 256: one of them in each part
+        if (D16 != 4 * DEC_PART + 4) return RA_ERR_ARG;
+        hipLaunchKernelGGL((attn_decode_kernel<4 * DEC_PART + 4, true>), grid, dim3(64), 0, st, q, pa, pm, kp, vp,
+                           pt, cup, kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz);
+        return RA_OK;
+    }
 #define DEC_CASE(N)                                                                                \
     case N:                                                                                        \
-        hipLaunchKernelGGL(attn_decode_kernel<N>, grid, dim3(64), 0, st, q, pa, pm, kp, vp, pt, cup, \
-                           kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits); \
+        hipLaunchKernelGGL((attn_decode_kernel<N, false>), grid, dim3(64), 0, st, q, pa, pm, kp, vp, pt, cup, \
+                           kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz); \
         return RA_OK;
     switch (D16) {
         DEC_CASE(4 * DEC_PART + 1) DEC_CASE(4 * DEC_PART + 2) DEC_CASE(4 * DEC_PART + 3)
@@ -267,7 +460,7 @@ extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t s
 #define DEC_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm,        \
     const bf16* kp, const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq,   \
     const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,                 \
-    int split_tokens, int max_splits
+    int split_tokens, int max_splits, DecodeFused fz
 extern "C" int ra_dec_part_0(DEC_PART_ARGS);
 extern "C" int ra_dec_part_1(DEC_PART_ARGS);
 extern "C" int ra_dec_part_2(DEC_PART_ARGS);
@@ -311,6 +504,38 @@ __global__ __launch_bounds__(128) void attn_decode_combine_kernel(
 // part_acc: fp32 [n_dec, Hq, max_splits, D]; part_ml: fp32 [n_dec, Hq, max_splits, 2].
 // max_splits is the number of splits of the request with the most; requests with fewer leave
 // the rest untouched and the merge does not read it.
+static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const bf16* kp, const bf16* vp,
+                         const int* page_table, const int* cu_pages, const int* kv_start, const int* cu_q,
+                         const int* q_start, const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
+                         float scale, int window, int split_tokens, int max_splits, DecodeFused fz,
+                         hipStream_t st) {
+    if (n_dec <= 0) return RA_OK;
+    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 ||
+        split_tokens <= 0 || split_tokens % DEC_CHUNK != 0 || max_splits <= 0 || max_splits > 65535 || P <= 0)
+        return RA_ERR_ARG;
+    const int head_blocks = Hkv * ((Hq / Hkv + DEC_MAX_GROUP - 1) / DEC_MAX_GROUP);
+    if (head_blocks > 65535) return RA_ERR_ARG;
+    dim3 grid(n_dec, head_blocks, max_splits);
+    int rc;
+    const int d16 = D / 16;
+#define DEC_GO(N) rc = ra_dec_part_##N(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, \
+                                       q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz)
+    switch ((d16 - 1) / 4) {
+        case 0: DEC_GO(0); break;
+        case 1: DEC_GO(1); break;
+        case 2: DEC_GO(2); break;
+        case 3: DEC_GO(3); break;
+        default: return RA_ERR_ARG;
+    }
+#undef DEC_GO
+    if (rc != RA_OK) return rc;
+    if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
+    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128),
+                       (size_t)max_splits * sizeof(float), st, pa, pm, (bf16*)out, kv_start, cu_q,
+                       q_start, seg_ids, Hq, D, window, split_tokens, max_splits);
+    return ra_launch_status();
+}
+
 extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc, void* part_ml,
                                         const void* k_pool, const void* v_pool,
                                         const int* page_table, const int* cu_pages,
@@ -318,33 +543,30 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
                                         const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
                                         float scale, int window, int split_tokens, int max_splits,
                                         void* stream) {
-    if (n_dec <= 0) return RA_OK;
-    if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 ||
-        split_tokens <= 0 || split_tokens % DEC_CHUNK != 0 || max_splits <= 0 || max_splits > 65535 || P <= 0)
+    DecodeFused none = {};
+    return decode_launch((const bf16*)q, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
+                         (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
+                         Hkv, D, P, scale, window, split_tokens, max_splits, none, (hipStream_t)stream);
+}
+
+// The same for requests whose new token has not been prepared: qkv [tokens, (Hq + 2 Hkv) D] as the
+// projection left it. The kernel norms (w_q, w_k [D]; nullptr: no norm) and rotates (cos, sin
+// [positions, D/2] at the request's position; nullptr: no rotation) q and k itself and writes k and
+// v of the new token into the pools. Head sizes 64, 128, 192, 256.
+extern "C" int ra_attention_decode_fused_bf16(const void* qkv, void* out, void* part_acc, void* part_ml,
+                                              void* k_pool, void* v_pool, const int* page_table,
+                                              const int* cu_pages, const int* kv_start, const int* cu_q,
+                                              const int* q_start, const int* seg_ids, int n_dec, int Hq,
+                                              int Hkv, int D, int P, float scale, int window,
+                                              int split_tokens, int max_splits, const float* w_q,
+                                              const float* w_k, float eps, const float* cos_t,
+                                              const float* sin_t, void* stream) {
+    if (qkv == nullptr || D % 64 != 0 || (w_q == nullptr) != (w_k == nullptr) ||
+        (cos_t == nullptr) != (sin_t == nullptr))
         return RA_ERR_ARG;
-    const int head_blocks = Hkv * ((Hq / Hkv + DEC_MAX_GROUP - 1) / DEC_MAX_GROUP);
-    if (head_blocks > 65535) return RA_ERR_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    dim3 grid(n_dec, head_blocks, max_splits);
-    const bf16* qq = (const bf16*)q;
-    const bf16* kp = (const bf16*)k_pool;
-    const bf16* vp = (const bf16*)v_pool;
-    float* pa = (float*)part_acc;
-    float* pm = (float*)part_ml;
-    int rc;
-    const int d16 = D / 16;
-    switch ((d16 - 1) / 4) {
-        case 0: rc = ra_dec_part_0(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        case 1: rc = ra_dec_part_1(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        case 2: rc = ra_dec_part_2(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        case 3: rc = ra_dec_part_3(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits); break;
-        default: return RA_ERR_ARG;
-    }
-    if (rc != RA_OK) return rc;
-    if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
-    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128),
-                       (size_t)max_splits * sizeof(float), st, pa, pm, (bf16*)out, kv_start, cu_q,
-                       q_start, seg_ids, Hq, D, window, split_tokens, max_splits);
-    return ra_launch_status();
+    DecodeFused fz = {(const bf16*)qkv, w_q, w_k, eps, cos_t, sin_t, (bf16*)k_pool, (bf16*)v_pool};
+    return decode_launch(nullptr, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
+                         (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
+                         Hkv, D, P, scale, window, split_tokens, max_splits, fz, (hipStream_t)stream);
 }
 #endif  // DEC_API

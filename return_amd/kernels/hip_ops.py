@@ -66,6 +66,7 @@ def _declare(lib):
         "ra_gemm_resident_fits": [I, I, I],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
+        "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, P],
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "ra_attention_prefill_tile_rows": [I],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
@@ -494,20 +495,7 @@ class HipOps:
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
         fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
         if fast_decode:
-            longest = step.max_decode_seq_len
-            S = self.decode_split_tokens
-            if S <= 0:
-                # about two thousand waves in all (eight per CU) fill the chip; fewer, longer
-                # splits spend less on starting up and on the merge (measured from 1 to 128 requests)
-                chunks = step.n_decode * n_kv * ((longest + 63) // 64)
-                S = 64 * max(2, -(-chunks // 2048), -(-longest // 4096))     # and at most 64 splits a request
-                if getattr(step, "decode_len_is_bound", False):
-                    # the lengths lie somewhere below `longest` (a graph's context bucket): splits
-                    # of at most an eighth of it keep the work of a request even
-                    S = min(S, max(128, longest // 8 // 64 * 64))
-            max_splits = (longest - 1) // S + 1
-            if window > 0:                       # a window spans at most this many splits
-                max_splits = min(max_splits, (window + S - 2) // S + 1)
+            S, max_splits = self._decode_splits(step, n_kv, window)
             nd = step.n_decode
             part_acc = torch.empty(nd, n_q, max_splits, D, dtype=torch.float32, device=self.device)
             part_ml = torch.empty(nd, n_q, max_splits, 2, dtype=torch.float32, device=self.device)
@@ -535,6 +523,67 @@ class HipOps:
         self._check(self.lib.ra_attention_plain(
             _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
             n_q, n_kv, D, P, float(scale), window, _code(q.dtype), self._stream()), "attention_plain")
+
+    def _decode_splits(self, step, n_kv, window):
+        """Keys per split of the decode attention and the most splits a request has."""
+        longest = step.max_decode_seq_len
+        S = self.decode_split_tokens
+        if S <= 0:
+            # about two thousand waves in all (eight per CU) fill the chip; fewer, longer
+            # splits spend less on starting up and on the merge (measured from 1 to 128 requests)
+            chunks = step.n_decode * n_kv * ((longest + 63) // 64)
+            S = 64 * max(2, -(-chunks // 2048), -(-longest // 4096))     # and at most 64 splits a request
+            if getattr(step, "decode_len_is_bound", False):
+                # the lengths lie somewhere below `longest` (a graph's context bucket): splits
+                # of at most an eighth of it keep the work of a request even
+                S = min(S, max(128, longest // 8 // 64 * 64))
+        max_splits = (longest - 1) // S + 1
+        if window > 0:                       # a window spans at most this many splits
+            max_splits = min(max_splits, (window + S - 2) // S + 1)
+        return S, max_splits
+
+    def attention_qkv(self, qkv, out, k_pool, v_pool, step, group, scale, window, n_q, n_kv, D,
+                      w_q, w_k, eps, cos, sin, rotary_dim):
+        """Attention of a step in which every request brings one token, straight from the q/k/v
+        projection: the decode kernel norms and rotates q and k itself and writes k and v into
+        the cache, which saves the preparation kernel. Returns False, having done nothing, when
+        the step or the sizes are not such (then qkv_prepare and attention do the work)."""
+        if qkv.dtype != torch.bfloat16 or step.n_decode != step.n_seqs or step.n_prefill_tokens != 0:
+            return False
+        R = int(rotary_dim)
+        if D % 64 or D > 256 or R not in (0, D) or (w_q is None) != (w_k is None):
+            return False
+        self._want(qkv, "qkv", torch.bfloat16, 2)
+        self._want(out, "attention output", torch.bfloat16, 3)
+        T = qkv.shape[0]
+        g = step.groups[group]
+        self._pool_rows(k_pool, v_pool, n_kv, D, torch.bfloat16)
+        if qkv.shape[1] != (n_q + 2 * n_kv) * D or tuple(out.shape) != (T, n_q, D) or T != step.n_tokens or n_q % n_kv:
+            raise KernelError(f"attention_qkv: qkv {tuple(qkv.shape)}, out {tuple(out.shape)}, "
+                              f"{n_q} heads over {n_kv} of {D}, step of {step.n_tokens}")
+        if w_q is not None:
+            for w in (w_q, w_k):
+                self._want(w, "head norm weight", torch.float32, 1)
+                if w.shape[0] != D:
+                    raise KernelError(f"attention_qkv: norm weight {tuple(w.shape)} for head size {D}")
+        if R:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if cos.shape[1] != D // 2 or sin.shape != cos.shape:
+                raise KernelError(f"attention_qkv: tables {tuple(cos.shape)} for head size {D}")
+        P = k_pool.shape[1]
+        window = int(window)
+        S, max_splits = self._decode_splits(step, n_kv, window)
+        nd = step.n_decode
+        part_acc = torch.empty(nd, n_q, max_splits, D, dtype=torch.float32, device=self.device)
+        part_ml = torch.empty(nd, n_q, max_splits, 2, dtype=torch.float32, device=self.device)
+        self._check(self.lib.ra_attention_decode_fused_bf16(
+            _ptr(qkv), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(k_pool), _ptr(v_pool),
+            _ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start),
+            _ptr(step.decode_segs), nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
+            _ptr(w_q), _ptr(w_k), float(eps), _ptr(cos) if R else None, _ptr(sin) if R else None,
+            self._stream()), "attention_decode_fused_bf16")
+        return True
 
     @staticmethod
     def _prefill_key_split(step, rows, n_workgroups):

@@ -65,6 +65,14 @@ class PagedAttention:
         T, Hq, Hkv, D = x.shape[0], self.n_q, self.n_kv, self.d
         tables = step.groups[cache.group]
         qkv = ops.linear(x, self.w_qkv)                              # [T, (Hq+2Hkv)*D]
+        if self._fusable and write_cache and hasattr(ops, "attention_qkv"):
+            # every request brings one token: the kernel set may prepare q, k and v inside its attention
+            cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
+            o = rt.empty(T, Hq, D)
+            if ops.attention_qkv(qkv, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale,
+                                 int(self.window) if self.window else 0, Hq, Hkv, D, self.w_qn, self.w_kn,
+                                 float(self.eps) if self.eps is not None else 0.0, cos, sin, rot):
+                return ops.linear(o.view(T, Hq * D), self.w_o)
         q = rt.empty(T, Hq, D)
         if self._fusable:
             cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)

@@ -523,6 +523,51 @@ def test_attention_far_key_stands_out(ops, dtype):
     torch.testing.assert_close(out[0, ::2].float(), want, atol=3e-2, rtol=3e-2)
 
 
+@pytest.mark.parametrize("split", [0, 64, 192])
+@pytest.mark.parametrize("D,Hq,Hkv,normed,rotated,window", [
+    (128, 8, 2, True, True, 0), (64, 4, 4, True, True, 0), (192, 3, 1, False, True, 0), (256, 4, 2, True, False, 0),
+    (128, 40, 2, True, True, 0), (64, 6, 2, True, True, 70), (128, 4, 1, False, False, 0)])
+def test_decode_attention_that_prepares_q_k_v_itself(ops, monkeypatch, D, Hq, Hkv, normed, rotated, window, split):
+    """The decode kernel fed with the projection's output (it norms and rotates q and k and writes
+    k and v into the cache) against the preparation kernel followed by the decode kernel: new
+    tokens at the first place, at the edges of pages, passes and splits, and far out."""
+    monkeypatch.setattr(ops, "decode_split_tokens", split)
+    P = 16
+    starts = [0, 1, 15, 16, 63, 64, 65, 127, 128, 191, 192, 700]
+    need = [-(-(a + 1) // P) for a in starts]
+    perm = torch.randperm(sum(need) + 3, generator=torch.Generator().manual_seed(D)).tolist()
+    pages_of = [[perm.pop() for _ in range(k)] for k in need]
+    step = _step([1] * len(starts), starts, P, pages_of)
+    n = len(starts)
+    kp = rnd(sum(need) + 3, P, Hkv, D, dtype=torch.bfloat16, seed=1)
+    vp = rnd(sum(need) + 3, P, Hkv, D, dtype=torch.bfloat16, seed=2)
+    qkv = rnd(n, (Hq + 2 * Hkv) * D, dtype=torch.bfloat16, seed=3)
+    wq = (1 + 0.1 * rnd(D, seed=4)) if normed else None
+    wk = (1 + 0.1 * rnd(D, seed=5)) if normed else None
+    pos = torch.arange(1024, device=DEV)[:, None] * (1.0 / 10000 ** (torch.arange(D // 2, device=DEV) / (D // 2)))[None]
+    cos, sin = (pos.cos().contiguous(), pos.sin().contiguous()) if rotated else (None, None)
+    R = D if rotated else 0
+    positions = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    slots = torch.tensor([pages_of[i][a // P] * P + a % P for i, a in enumerate(starts)], dtype=torch.int32, device=DEV)
+    # two kernels
+    k1, v1 = kp.clone(), vp.clone()
+    q = torch.zeros(n, Hq, D, dtype=torch.bfloat16, device=DEV)
+    ops.qkv_prepare(qkv, Hq, Hkv, D, wq, wk, 1e-5, positions, cos, sin, R, q, k1, v1, slots)
+    want = torch.zeros_like(q)
+    ops.attention(q, want, k1, v1, step, 0, D ** -0.5, window)
+    # one kernel
+    k2, v2 = kp.clone(), vp.clone()
+    got = torch.zeros_like(q)
+    assert ops.attention_qkv(qkv, got, k2, v2, step, 0, D ** -0.5, window, Hq, Hkv, D, wq, wk, 1e-5, cos, sin, R)
+    assert torch.equal(v1, v2)                                         # values are copied
+    torch.testing.assert_close(k2.float(), k1.float(), atol=0, rtol=2 ** -7)      # keys: the last bit of the rounding at most
+    assert (k2 != k1).float().mean().item() < 1e-3
+    torch.testing.assert_close(got.float(), want.float(), **tol(torch.bfloat16))
+    # a step with a portion in it is not taken
+    mixed = _step([1, 3], [5, 0], P, [[0], [1]])
+    assert not ops.attention_qkv(qkv[:4], got[:4], k2, v2, mixed, 0, 1.0, 0, Hq, Hkv, D, wq, wk, 1e-5, cos, sin, R)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_over_a_long_context(ops, ref, dtype):
     """40,000 keys in scattered pages: a decoded token at the end of them, one after five keys, and
