@@ -54,7 +54,7 @@ class Engine:
         self.scheduler = Scheduler(runner.cache, ec.max_reside, ec.max_step_tokens, ec.prefill_chunk,
                                    runner.max_position)
         self._submitted = 0
-        self._in_flight = None              # (ticket, plan) of a decode step that was launched and not yet collected
+        self._in_flight = None              # (ticket, plan) of a step that was launched and not yet collected
         # running totals as in rollout/engine.py:84-125
         self.prefill_tokens = 0
         self.decode_tokens = 0
@@ -93,19 +93,29 @@ class Engine:
                 raise ValueError(f"{name}: prompt token {t} outside the vocabulary of {self.runner.vocab_size}")
 
     # ------------------------------------------------------------------ one step
-    def _launch_decode(self, plan, previous=None):
-        """Start a decode-only plan. previous: the plan whose sampled tokens, still on the device,
-        are this plan's tokens (its rows are looked up by request)."""
-        rows = [e.request for e in plan.entries]
-        if previous is None:
-            tokens, feed = [e.tokens[0] for e in plan.entries], None
-        else:
-            row_of = {e.request.id: i for i, e in enumerate(previous.entries)}
-            tokens, feed = None, [row_of[r.id] for r in rows]
-        return self.runner.decode_launch(
-            [r.id for r in rows], tokens, [r.params.temperature for r in rows],
-            [r.params.top_k for r in rows], [r.params.top_p for r in rows],
-            [r.stream.next() for r in rows], feed_rows=feed)
+    def _launch(self, plan, previous=None):
+        """Start a plan; returns the ticket to collect its sampled tokens with. previous: the plan
+        under way whose sampled tokens, still on the device, are the tokens of this plan's entries
+        that hold None (their rows among previous's sampled entries are looked up by request)."""
+        sampled = [e.request for e in plan.entries if e.sample]
+        options = ([r.params.temperature for r in sampled], [r.params.top_k for r in sampled],
+                   [r.params.top_p for r in sampled], [r.stream.next() for r in sampled])
+        row_of = {}
+        if previous is not None:
+            row_of = {e.request.id: i for i, e in enumerate(x for x in previous.entries if x.sample)}
+        if all(e.sample and len(e.tokens) == 1 for e in plan.entries):
+            # decode only: one call that runs the model and the sampler (from a graph if enabled)
+            unknown = [e.tokens[0] is None for e in plan.entries]
+            if any(unknown) and not all(unknown):
+                raise RuntimeError("a decode step takes either all or none of its tokens from the step before")
+            ids = [e.request.id for e in plan.entries]
+            if all(unknown):
+                return self.runner.decode_launch(ids, None, *options, feed_rows=[row_of[i] for i in ids])
+            return self.runner.decode_launch(ids, [e.tokens[0] for e in plan.entries], *options)
+        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
+                   for e in plan.entries]
+        feed = [(i, row_of[e.request.id]) for i, e in enumerate(plan.entries) if e.tokens[0] is None]
+        return self.runner.step_launch(entries, *options, feed=feed)
 
     def _book(self, plan, sampled, t0):
         for e in plan.entries:
@@ -125,48 +135,49 @@ class Engine:
         self.steps += 1
         return ended
 
+    def _collect(self, ticket, plan, t0):
+        sampled_entries = [e for e in plan.entries if e.sample]
+        sampled = {}
+        if sampled_entries:
+            toks, logps = self.runner.decode_collect(ticket)
+            sampled = {e.request.id: (t, lp) for e, t, lp in zip(sampled_entries, toks, logps)}
+        return self._book(plan, sampled, t0)
+
     def step(self) -> List[Request]:
         """One scheduler step; returns the requests that ended in it (finished or failed).
 
-        A decode-only step is launched and collected in two halves: while it runs, the step
-        after it is decided and launched if it can be decided without the tokens
-        (Scheduler.schedule_ahead), so that the device does not wait for the host between steps.
+        A step is launched and collected in two halves: while it runs, the step after it is
+        decided (Scheduler.schedule_ahead) and launched, its tokens taken over on the device, so
+        that the device does not wait for the host between steps.
         """
         t0 = time.perf_counter()
-        if self._in_flight is not None:
-            ticket, plan = self._in_flight
-            ahead = self.scheduler.schedule_ahead(plan) if self.config.lookahead else None
-            next_ticket = self._launch_decode(ahead, previous=plan) if ahead is not None else None
-            toks, logps = self.runner.decode_collect(ticket)
-            sampled = {e.request.id: (t, lp) for e, t, lp in zip(plan.entries, toks, logps)}
-            ended = self._book(plan, sampled, t0)
-            self._in_flight = (next_ticket, ahead) if ahead is not None else None
-            return ended
-        plan = self.scheduler.schedule()
-        ended = list(plan.failed)
-        if not plan.entries:
-            return ended
-        if all(e.sample and len(e.tokens) == 1 for e in plan.entries):
-            # decode only: one call that runs the model and the sampler (from a graph if enabled)
-            ticket = self._launch_decode(plan)
-            if self.config.lookahead:
-                self._in_flight = (ticket, plan)
-                return ended + self.step()
-            toks, logps = self.runner.decode_collect(ticket)
-            sampled = {e.request.id: (t, lp) for e, t, lp in zip(plan.entries, toks, logps)}
-            return ended + self._book(plan, sampled, t0)
-        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
-                   for e in plan.entries]
-        logits = self.runner.step(entries)
-        rows = [e.request for e in plan.entries if e.sample]
-        sampled: Dict[object, tuple] = {}
-        if rows:
-            toks, logps = self.runner.sample(
-                logits, [r.params.temperature for r in rows], [r.params.top_k for r in rows],
-                [r.params.top_p for r in rows], [r.stream.next() for r in rows])
-            for r, t, lp in zip(rows, toks, logps):
-                sampled[r.id] = (t, lp)
-        return ended + self._book(plan, sampled, t0)
+        ended: List[Request] = []
+        if self._in_flight is None:
+            plan = self.scheduler.schedule()
+            ended += plan.failed
+            if not plan.entries:
+                return ended
+            ticket = self._launch_or_run(plan)
+            if not self.config.lookahead:
+                return ended + self._collect(ticket, plan, t0)
+            self._in_flight = (ticket, plan)
+        ticket, plan = self._in_flight
+        ahead = self.scheduler.schedule_ahead(plan) if self.config.lookahead else None
+        following = None
+        if ahead is not None:
+            ended += ahead.failed
+            if ahead.entries:
+                following = (self._launch_or_run(ahead, previous=plan), ahead)
+        ended += self._collect(ticket, plan, t0)
+        self._in_flight = following
+        return ended
+
+    def _launch_or_run(self, plan, previous=None):
+        """_launch, or for a plan in which nothing is sampled (prompt portions only) the plain step."""
+        if any(e.sample for e in plan.entries):
+            return self._launch(plan, previous)
+        self.runner.step([StepEntry(e.request.id, e.tokens, []) for e in plan.entries])
+        return None
 
     # ------------------------------------------------------------------ whole jobs
     def generate(self, prompts: Sequence[Sequence[int]],

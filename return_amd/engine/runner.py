@@ -81,6 +81,8 @@ class ModelRunner:
         self._picked_ready = [torch.cuda.Event() if pin else None for _ in range(2)]
         self._feed_host = torch.zeros(n, dtype=torch.int64, pin_memory=pin)
         self._feed_dev = torch.zeros(n, dtype=torch.int64, device=self.rt.device)
+        self._feed_at_host = torch.zeros(n, dtype=torch.int64, pin_memory=pin)
+        self._feed_at_dev = torch.zeros(n, dtype=torch.int64, device=self.rt.device)
         self._launches = 0
         self._last_picked: Optional[torch.Tensor] = None
 
@@ -103,6 +105,11 @@ class ModelRunner:
         """
         if not entries:
             return None
+        return self._run(entries, None)[0]
+
+    def _run(self, entries: Sequence[StepEntry], after_build):
+        """Checks, cache tables, device tables, forward. after_build(batch) runs between the copy
+        of the tables and the model. Returns (logits or None, batch)."""
         rows: List[int] = []
         at = 0
         for e in entries:
@@ -110,7 +117,7 @@ class ModelRunner:
             if n == 0:
                 raise ValueError(f"request {e.request_id!r} brings no tokens")
             for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
+                if t is not None and not 0 <= int(t) < self.vocab_size:
                     raise ValueError(f"request {e.request_id!r}: token {t} outside the vocabulary of {self.vocab_size}")
             if e.request_id in self.cache.live and self.cache.seq_len(e.request_id) + n > self.max_position:
                 raise ValueError(
@@ -123,12 +130,65 @@ class ModelRunner:
             at += n
         tables = self.cache.begin_step([(e.request_id, len(e.tokens)) for e in entries])
         try:
-            batch = self.builder.build(tables, [e.tokens for e in entries], rows)
+            batch = self.builder.build(tables, [[0 if t is None else t for t in e.tokens] for e in entries], rows)
+            if after_build is not None:
+                after_build(batch)
             with torch.no_grad():
                 logits = self.model.forward(batch, self.cache)
         finally:
             self.cache.end_step()
-        return logits
+        return logits, batch
+
+    def step_launch(self, entries: Sequence[StepEntry], temperature, top_k, top_p, uniforms, feed=None):
+        """Start a step of any kind whose wanted places are all sampled, and return a ticket for
+        decode_collect. Nothing here waits for the device.
+
+        A token may be None in an entry of one token: then feed lists (entry number, row of the
+        previous launch's sampled tokens) and the token is taken from there on the device, so
+        that this step can be launched before the previous one's tokens have been read.
+        temperature, top_k, top_p, uniforms: one per wanted place, in the entries' order.
+        """
+        m = sum(len(e.want) for e in entries)
+        if m == 0 or m > self.engine_config.max_reside or len(temperature) != m:
+            raise ValueError(f"step_launch: {m} sampled places, {len(temperature)} sampling options, "
+                             f"at most {self.engine_config.max_reside}")
+        feed = list(feed or [])
+        fed = {i for i, _ in feed}
+        for i, e in enumerate(entries):
+            if (None in e.tokens) != (i in fed) or (i in fed and len(e.tokens) != 1):
+                raise ValueError("step_launch: tokens that are None and the list of rows to take them from do not match")
+        if feed and (self._last_picked is None or
+                     any(not 0 <= int(r) < self._last_picked.shape[0] for _, r in feed)):
+            raise ValueError("step_launch: a row to take a token from is not a row of the previous launch")
+
+        def take_tokens(batch):
+            if feed:
+                if self._samp_copied is not None:
+                    self._samp_copied.synchronize()      # the last launch's copies have left the staging buffers
+                k = len(feed)
+                starts = batch.cu_q_host
+                self._feed_host[:k] = torch.as_tensor([int(r) for _, r in feed], dtype=torch.int64)
+                self._feed_at_host[:k] = torch.as_tensor([starts[i] for i, _ in feed], dtype=torch.int64)
+                self._feed_dev[:k].copy_(self._feed_host[:k], non_blocking=True)
+                self._feed_at_dev[:k].copy_(self._feed_at_host[:k], non_blocking=True)
+                batch.token_ids.index_copy_(0, self._feed_at_dev[:k],
+                                            self._last_picked[:, 0].index_select(0, self._feed_dev[:k]))
+            self._put_sampling(m, temperature, top_k, top_p, uniforms)
+
+        logits, _ = self._run(entries, take_tokens)
+        with torch.no_grad():
+            picked = self.rt.ops.sample(logits, self._samp_dev_f[0, :m], self._samp_dev_k[:m],
+                                        self._samp_dev_f[1, :m], self._samp_dev_f[2, :m])
+        return self._ticket(picked, m, logits)
+
+    def _ticket(self, picked, n, logits):
+        slot = self._launches & 1
+        self._launches += 1
+        self._last_picked = picked
+        self._picked_host[slot][:n].copy_(picked[:n], non_blocking=True)
+        if self._picked_ready[slot] is not None:
+            self._picked_ready[slot].record()
+        return (slot, n, logits[:n])
 
     # ------------------------------------------------------------------ decode from a graph
     def _put_sampling(self, m, temperature, top_k, top_p, uniforms):
@@ -183,6 +243,8 @@ class ModelRunner:
             batch = self.builder.build(tables, host_tokens, list(range(rows)))
             if tokens is None:
                 # after the tables' copy and before the step: the sampled tokens become the new tokens
+                if self._samp_copied is not None:
+                    self._samp_copied.synchronize()      # the last launch's copies have left the staging buffers
                 self._feed_host[:n] = torch.as_tensor(list(feed_rows), dtype=torch.int64)
                 self._feed_dev[:n].copy_(self._feed_host[:n], non_blocking=True)
                 batch.token_ids[:n].copy_(self._last_picked[:, 0].index_select(0, self._feed_dev[:n]))
@@ -196,13 +258,7 @@ class ModelRunner:
                     logits, picked = self._decode_body(batch)
         finally:
             self.cache.end_step()
-        slot = self._launches & 1
-        self._launches += 1
-        self._last_picked = picked
-        self._picked_host[slot][:n].copy_(picked[:n], non_blocking=True)
-        if self._picked_ready[slot] is not None:
-            self._picked_ready[slot].record()
-        return (slot, n, logits[:n])
+        return self._ticket(picked, n, logits)
 
     def decode_collect(self, ticket):
         """Wait for a launched decode step; returns (tokens, logprobs) as Python lists."""

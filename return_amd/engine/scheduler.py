@@ -203,25 +203,58 @@ class Scheduler:
     # ------------------------------------------------------------------ one step
     def schedule(self) -> StepPlan:
         """Decide the next step: one token of every decoding request, then prompt portions."""
+        return self._plan({})
+
+    def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
+        """The step after ``plan``, decided while plan is still under way and its sampled tokens
+        are not known: the same decisions as schedule(), taken on the state that plan will leave.
+        A request that samples in plan decodes next; its token is None here (it is still on the
+        device) unless that token is its last (max_new_tokens), then it is left out. A request
+        that ends on a stop sequence in plan is found out only later: finish_step then skips its
+        entry in the step returned here (the token computed for it is dropped, its pages go back
+        with the request). What plan's finished requests hold is given back only when plan is
+        booked, so a newcomer may be let in one step later than without looking ahead.
+        None: there is nothing to run."""
+        under_way = {e.request.id: e for e in plan.entries if not e.request.finished}
+        ahead = self._plan(under_way)
+        return ahead if ahead.entries or ahead.failed else None
+
+    def _plan(self, under_way: Dict[object, PlannedEntry]) -> StepPlan:
+        """under_way: entries of a step that runs but is not booked yet, by request."""
         budget = self.max_step_tokens
         entries: List[PlannedEntry] = []
         failed: List[Request] = []
 
-        def take(r: Request, limit: int):
+        def state(r: Request):
+            e = under_way.get(r.id)
+            computed = r.num_computed + (len(e.tokens) if e is not None else 0)
+            outputs = len(r.output) + (1 if e is not None and e.sample else 0)
+            return computed, outputs, e
+
+        def portion(r: Request, computed: int):
             nonlocal budget
-            pend = r.pending()
-            n = min(len(pend), limit, budget)
+            n_prompt = len(r.prompt_ids)
+            n = min(n_prompt - computed, self.prefill_chunk, budget)
             if n <= 0:
                 return
-            entries.append(PlannedEntry(r, pend[:n], sample=(n == len(pend))))
+            entries.append(PlannedEntry(r, r.prompt_ids[computed:computed + n], sample=(computed + n == n_prompt)))
             budget -= n
 
         for r in self.running:                      # decoding requests first
-            if r.num_computed >= len(r.prompt_ids):
-                take(r, 1)
+            computed, outputs, e = state(r)
+            if computed < len(r.prompt_ids) or budget <= 0:
+                continue
+            if e is not None and e.sample:
+                if outputs >= r.max_new:            # the step under way brings its last token
+                    continue
+                entries.append(PlannedEntry(r, [None], sample=True))
+            else:
+                entries.append(PlannedEntry(r, [r.output[-1]], sample=True))
+            budget -= 1
         for r in self.running:                      # prompts under way
-            if r.num_computed < len(r.prompt_ids):
-                take(r, self.prefill_chunk)
+            computed, _, _ = state(r)
+            if computed < len(r.prompt_ids):
+                portion(r, computed)
         while self.waiting and budget > 0:          # newcomers, in order
             r = self.waiting[0]
             ok = self._try_admit(r)
@@ -232,25 +265,8 @@ class Scheduler:
             if not ok:
                 break
             self.waiting.popleft()
-            take(r, self.prefill_chunk)
+            portion(r, r.num_computed)
         return StepPlan(entries, failed)
-
-    def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
-        """The step after ``plan``, decided before plan's sampled tokens are known. That is
-        possible only when nothing but the tokens themselves is missing: plan is one token of
-        every running request and nobody waits. Requests for which plan's token is the last
-        (max_new_tokens) are left out. A request that ends on a stop sequence in ``plan`` is
-        found out only later; finish_step then skips its entry in the step returned here (the
-        token it computed is dropped, its pages go back with the request). The tokens of the
-        entries are None: they are still on the device."""
-        live = [e for e in plan.entries if not e.request.finished]
-        if self.waiting or len(live) != len(self.running):
-            return None
-        if any(len(e.tokens) != 1 or not e.sample for e in live):
-            return None
-        entries = [PlannedEntry(e.request, [None], sample=True) for e in live
-                   if len(e.request.output) + 1 < e.request.max_new]
-        return StepPlan(entries, []) if entries else None
 
     def finish_step(self, plan: StepPlan, sampled: Dict[object, Tuple[int, float]]) -> List[Request]:
         """Book the step: tokens are in the cache, sampled tokens join the outputs. Returns who finished."""

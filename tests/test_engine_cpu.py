@@ -161,24 +161,39 @@ def test_steps_launched_ahead_give_the_same_generation(folder_a):
     assert eng.decode_tokens == sum(len(o) - 1 for o, _, _ in plain_run)    # a dropped token is not counted
 
 
-def test_schedule_ahead_only_when_the_tokens_are_all_that_is_missing(folder_a):
+def test_schedule_ahead_decides_on_the_state_the_step_under_way_will_leave(folder_a):
     from return_amd.engine.scheduler import Request, Scheduler
     runner = runner_for(folder_a, 512, max_reside=3)
     sch = Scheduler(runner.cache, 3, 64, 32, runner.max_position)
     a = Request("a", [1, 2, 3], SamplingParams(max_new_tokens=3))
-    b = Request("b", [4, 5], SamplingParams(max_new_tokens=2))
+    b = Request("b", list(range(40)), SamplingParams(max_new_tokens=2))
     sch.add(a); sch.add(b)
-    plan = sch.schedule()                                    # both prompts whole
-    assert sch.schedule_ahead(plan) is None                  # not a decode step
-    sch.finish_step(plan, {"a": (7, 0.0), "b": (8, 0.0)})
-    for r, n in ((a, 3), (b, 2)):                            # the runner's side of the step
-        runner.cache.begin_step([(r.id, n)]); runner.cache.end_step()
-    plan = sch.schedule()
-    assert [e.tokens for e in plan.entries] == [[7], [8]]
-    ahead = sch.schedule_ahead(plan)                         # b's second token is its last: only a goes on
-    assert [e.request.id for e in ahead.entries] == ["a"] and ahead.entries[0].tokens == [None]
-    sch.add(Request("c", [9], SamplingParams(max_new_tokens=2)))
-    assert sch.schedule_ahead(plan) is None                  # somebody waits: the next step is not only decoding
+
+    def run(plan):                                           # the runner's side of a step
+        runner.cache.begin_step([(e.request.id, len(e.tokens)) for e in plan.entries]); runner.cache.end_step()
+
+    plan = sch.schedule()                                    # a's prompt whole, b's first portion
+    assert [(e.request.id, len(e.tokens), e.sample) for e in plan.entries] == [("a", 3, True), ("b", 32, False)]
+    run(plan)
+    ahead = sch.schedule_ahead(plan)                         # a decodes a token nobody knows yet, b's prompt ends
+    assert [(e.request.id, e.tokens if e.request is a else len(e.tokens), e.sample) for e in ahead.entries] == \
+        [("a", [None], True), ("b", 8, True)]
+    assert a.num_computed == 0 and not a.output              # nothing is booked by looking ahead
+    sch.finish_step(plan, {"a": (7, 0.0)})
+    run(ahead)
+    sch.add(Request("c", [9, 9], SamplingParams(max_new_tokens=2)))
+    ahead2 = sch.schedule_ahead(ahead)                       # both decode, the newcomer is let in
+    assert [(e.request.id, e.tokens) for e in ahead2.entries] == [("a", [None]), ("b", [None]), ("c", [9, 9])]
+    sch.finish_step(ahead, {"a": (8, 0.0), "b": (5, 0.0)})
+    run(ahead2)
+    ahead3 = sch.schedule_ahead(ahead2)                      # a's and b's tokens of ahead2 are their last: only c goes on
+    assert [(e.request.id, e.tokens) for e in ahead3.entries] == [("c", [None])]
+    done = sch.finish_step(ahead2, {"a": (1, 0.0), "b": (2, 0.0), "c": (3, 0.0)})
+    assert {r.id for r in done} == {"a", "b"} and a.output == [7, 8, 1] and b.output == [5, 2]
+    run(ahead3)
+    assert sch.schedule_ahead(ahead3) is None                # c's token of ahead3 is its last: nothing is left to run
+    sch.finish_step(ahead3, {"c": (4, 0.0)})
+    assert not sch.has_work() and not runner.cache.live
 
 
 def engine_for(folder, lookahead=True, **kw):
@@ -264,3 +279,35 @@ def test_kept_sessions_that_do_not_fit_or_do_not_match(folder_a):
     while eng.scheduler.has_work() or eng._in_flight is not None:
         eng.step()
     assert r.finish_reason == "length" and not eng.runner.cache.live
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_launching_ahead_never_changes_what_is_generated(folder_a, seed):
+    """Random prompts, lengths, stop sequences and knobs: with every step launched before the one
+    before it is collected (prompt portions beside decoded tokens included) the outputs and finish
+    reasons equal the plain implementation's, and nothing is left in the cache."""
+    import random
+    rnd = random.Random(seed)
+    cfg, w = plain.read_folder(folder_a)
+    V = TINY_A["vocab_size"]
+    n = rnd.randint(3, 9)
+    prompts = [tt.random_tokens(V, rnd.randint(1, 90), seed=seed * 100 + i) for i in range(n)]
+    news = [rnd.randint(1, 12) for _ in range(n)]
+    stops = []
+    for p, k in zip(prompts, news):
+        free = plain.greedy_generate(cfg, w, p, k)
+        stops.append([free[j:j + 2]] if k >= 4 and rnd.random() < 0.5 and (j := rnd.randint(0, k - 2)) >= 0 else [])
+    want = [plain.greedy_generate(cfg, w, p, k, stop_ids=s) for p, k, s in zip(prompts, news, stops)]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=k, stop_ids=s) for k, s in zip(news, stops)]
+    max_reside = rnd.randint(1, 5)
+    eng = engine_for(folder_a, True, max_reside=max_reside, max_token=rnd.choice([256, 512, 2048]))
+    eng.config.prefill_chunk = eng.scheduler.prefill_chunk = rnd.choice([5, 24, 64])
+    launches = []
+    inner = eng._launch_or_run
+    eng._launch_or_run = lambda plan, previous=None: (launches.append(previous is not None), inner(plan, previous))[1]
+    out = eng.generate(prompts, params)
+    assert [r.output_ids for r in out] == want
+    assert [r.finish_reason for r in out] == ["stop" if s and o[-2:] == s[0] else "length" for o, s in zip(want, stops)]
+    assert any(launches) and eng._in_flight is None           # steps were launched ahead
+    eng.runner.cache.check_invariants()
+    assert not eng.runner.cache.live and all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
