@@ -103,11 +103,10 @@ class Engine:
         row_of = {}
         if previous is not None:
             row_of = {e.request.id: i for i, e in enumerate(x for x in previous.entries if x.sample)}
-        if all(e.sample and len(e.tokens) == 1 for e in plan.entries):
-            # decode only: one call that runs the model and the sampler (from a graph if enabled)
-            unknown = [e.tokens[0] is None for e in plan.entries]
-            if any(unknown) and not all(unknown):
-                raise RuntimeError("a decode step takes either all or none of its tokens from the step before")
+        unknown = [e.tokens[0] is None for e in plan.entries]
+        if all(e.sample and len(e.tokens) == 1 for e in plan.entries) and (all(unknown) or not any(unknown)):
+            # one token each (decoded tokens, or prompts of one token), all known or all still on the
+            # device: one call that runs the model and the sampler (from a graph if enabled)
             ids = [e.request.id for e in plan.entries]
             if all(unknown):
                 return self.runner.decode_launch(ids, None, *options, feed_rows=[row_of[i] for i in ids])

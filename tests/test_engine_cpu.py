@@ -311,3 +311,21 @@ def test_launching_ahead_never_changes_what_is_generated(folder_a, seed):
     assert any(launches) and eng._in_flight is None           # steps were launched ahead
     eng.runner.cache.check_invariants()
     assert not eng.runner.cache.live and all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+
+
+def test_a_prompt_of_one_token_beside_tokens_that_are_still_on_the_device(folder_a):
+    """A newcomer whose prompt is a single token joins a step whose other tokens are not known
+    yet: one token each, but not a step that takes all its tokens from the step before."""
+    cfg, w = plain.read_folder(folder_a)
+    V = TINY_A["vocab_size"]
+    eng = engine_for(folder_a, True, max_reside=4)
+    sp = SamplingParams(temperature=0.0, max_new_tokens=8)
+    first = [eng.submit(tt.random_tokens(V, n, seed=n), sp) for n in (7, 20)]
+    for _ in range(3):
+        eng.step()
+    late = [eng.submit([5], sp), eng.submit([9], SamplingParams(temperature=0.0, max_new_tokens=1))]
+    while eng.scheduler.has_work() or eng._in_flight is not None:
+        eng.step()
+    for r in first + late:
+        assert r.output == plain.greedy_generate(cfg, w, r.prompt_ids, r.max_new)
+    assert not eng.runner.cache.live
