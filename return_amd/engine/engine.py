@@ -172,11 +172,19 @@ class Engine:
         return ended
 
     def _launch_or_run(self, plan, previous=None):
-        """_launch, or for a plan in which nothing is sampled (prompt portions only) the plain step."""
-        if any(e.sample for e in plan.entries):
-            return self._launch(plan, previous)
-        self.runner.step([StepEntry(e.request.id, e.tokens, []) for e in plan.entries])
-        return None
+        """_launch, or for a plan in which nothing is sampled (prompt portions only) the plain step.
+        If the step cannot be started, its requests fail with the error (what they hold goes back,
+        as in the reference's _fail, rollout/engine.py:317-324) and the error is raised."""
+        try:
+            if any(e.sample for e in plan.entries):
+                return self._launch(plan, previous)
+            self.runner.step([StepEntry(e.request.id, e.tokens, []) for e in plan.entries])
+            return None
+        except Exception as error:
+            for e in plan.entries:
+                if not e.request.finished:
+                    self.scheduler.abort(e.request, error)
+            raise
 
     # ------------------------------------------------------------------ whole jobs
     def generate(self, prompts: Sequence[Sequence[int]],

@@ -50,14 +50,6 @@ class Request:
     def num_tokens(self) -> int:
         return len(self.prompt_ids) + len(self.output)
 
-    def pending(self) -> List[int]:
-        """Tokens not yet in the cache: the rest of the prompt, or the last sampled token."""
-        k = self.num_computed
-        n_prompt = len(self.prompt_ids)
-        if k < n_prompt:
-            return self.prompt_ids[k:] + self.output
-        return self.output[k - n_prompt:]
-
     @property
     def finished(self) -> bool:
         return self.status in ("finished", "failed")

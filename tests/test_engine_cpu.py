@@ -329,3 +329,24 @@ def test_a_prompt_of_one_token_beside_tokens_that_are_still_on_the_device(folder
     for r in first + late:
         assert r.output == plain.greedy_generate(cfg, w, r.prompt_ids, r.max_new)
     assert not eng.runner.cache.live
+
+
+def test_a_step_that_cannot_start_fails_its_requests_and_frees_them(folder_a, monkeypatch):
+    eng = engine_for(folder_a, True, max_reside=4)
+    sp = SamplingParams(temperature=0.0, max_new_tokens=5)
+    a = eng.submit([1, 2, 3], sp)
+    eng.step()
+
+    def broken(*args, **kw):
+        raise RuntimeError("the device said no")
+    monkeypatch.setattr(eng.runner, "decode_launch", broken)
+    monkeypatch.setattr(eng.runner, "step_launch", broken)
+    b = eng.submit([4, 5], sp)
+    with pytest.raises(RuntimeError, match="said no"):
+        while eng.scheduler.has_work() or eng._in_flight is not None:
+            eng.step()
+    assert a.finish_reason == b.finish_reason == "error" and "said no" in str(a.error)
+    monkeypatch.undo()
+    out = eng.generate([[7, 8, 9]], sp)[0]                 # the step that was under way is collected, then life goes on
+    assert out.num_tokens == 5 and not eng.runner.cache.live
+    eng.runner.cache.check_invariants()
