@@ -19,7 +19,7 @@ class EngineConfig:
     max_step_tokens: int = 8192        # token budget of one step (decoded tokens + prompt portions)
     prefill_chunk: int = 8192          # longest portion of one prompt in one step
     use_graphs: bool = True            # replay decode-only steps from captured HIP graphs (USE_CUDA_GRAPH of the reference)
-    lookahead: bool = True             # launch the next decode step before this one's tokens are read
+    lookahead: bool = True             # launch every step before the sampled tokens of the one before it are read
     tune_products: bool = True         # measure at load which kernel forms each projection fastest at few rows
     seed: int = 0                      # base seed of the sampling streams
     device: str = "cuda:0"
