@@ -21,7 +21,7 @@ import sys
 
 import numpy as np
 
-MAX_LIVE = 4            # requests live at a time
+MAX_LIVE = 8            # request slots: traces keep up to four requests live, with room to spare
 ROUND_TO = 64           # a request's token count is rounded up to this for --max-tokens
 
 
@@ -40,8 +40,10 @@ def main(argv=None) -> int:
     os.makedirs(args.out, exist_ok=True)
     page = 16                                   # divides ROUND_TO, so the pool is exactly max-tokens
     pool = -(-args.max_tokens // ROUND_TO) * ROUND_TO
+    # products by rule, not by the measurement at load, whose choices may differ from run to run:
+    # two replays of a trace give the same bits
     ec = EngineConfig(dtype=args.dtype, page_size=page, max_token=pool, max_reside=MAX_LIVE,
-                      max_step_tokens=max(pool, MAX_LIVE), prefill_chunk=pool)
+                      max_step_tokens=max(pool, MAX_LIVE), prefill_chunk=pool, tune_products=False)
     runner = ModelRunner(args.model, engine_config=ec)
 
     for line in sys.stdin:

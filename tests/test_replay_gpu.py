@@ -88,6 +88,10 @@ def test_trace_run_program(folder_a, tmp_path, dtype):
     got = tt.run_program(folder_a, dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps),
                          TINY_A["vocab_size"])
     compare(got, want, reqs, dtype)
+    if dtype == "bfloat16":                      # a second replay gives the same bits
+        again = tt.run_program(folder_a, dtype, steps, str(tmp_path / "out2"), tt.peak_tokens(steps),
+                               TINY_A["vocab_size"])
+        assert got.keys() == again.keys() and all(torch.equal(got[k], again[k]) for k in got)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
