@@ -25,7 +25,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# BASELINE.json configs[2]: Qwen3-8B shape
+# the headline configuration: Qwen3-8B shape
 QWEN3_8B = dict(
     architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=151936, hidden_size=4096,
     num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
@@ -137,7 +137,7 @@ def release(runner, ids):
         runner.free_request(rid)
 
 
-# BASELINE.json configs[3] and configs[4]: the other two shapes, with the workloads named there
+# the two other shapes of the benchmark, each with its own workload
 QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64,
                  intermediate_size=25600)
