@@ -74,6 +74,14 @@ struct DecodeFused {
 };
 
 #ifdef DEC_PART
+// Order between the LDS accesses of one wave (a write by one lane, a read of it by another): LDS
+// serves a wave's instructions in order, so only the compiler has to keep them in order.
+#define WAVE_SYNC()                                              \
+    do {                                                         \
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");   \
+        __builtin_amdgcn_wave_barrier();                         \
+    } while (0)
+
 // two floats to two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
     const float2_t v = {a, b};
@@ -166,14 +174,26 @@ __device__ __forceinline__ void prepare_head(bf16x8_t (&v)[D32], const float* __
     else if (cs != nullptr) prepare_head_as<D32, false, true>(v, w, eps, cs, sn, g);
 }
 
+// LDS of one wave: its value tile, and after its passes its sums for the merge (whichever is larger)
+__host__ __device__ constexpr int dec_region_bytes(int D) {
+    return (DEC_CHUNK * (D + 16) * 2 > 16 * (D + 2) * 4) ? DEC_CHUNK * (D + 16) * 2 : 16 * (D + 2) * 4;
+}
+
+// merge_waves == 1: one wave per workgroup, blockIdx.z is the split, partial sums go to memory
+// and attn_decode_combine_kernel merges them. merge_waves > 1: a workgroup of merge_waves waves
+// per (request, kv head), wave w takes split w, and the waves' sums are merged through LDS here
+// (the same sums in the same order as the merge kernel), so that nothing goes through memory and
+// no second kernel runs; for requests whose splits fit one workgroup.
 template <int D16, bool FUSED>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2 : 1))) void attn_decode_kernel(
+__global__ __launch_bounds__(D16 <= 8 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2 : 1)))
+void attn_decode_kernel(
     const bf16* __restrict__ q, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const bf16* k_pool, const bf16* v_pool,
     const int* __restrict__ page_table, const int* __restrict__ cu_pages,
     const int* __restrict__ kv_start, const int* __restrict__ cu_q,
     const int* __restrict__ q_start, const int* __restrict__ seg_ids, int Hq, int Hkv, int P,
-    float scale, int window, int split_tokens, int max_splits, DecodeFused fz) {
+    float scale, int window, int split_tokens, int max_splits, DecodeFused fz, int merge_waves,
+    bf16* __restrict__ out) {
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;                 // full MFMA x32 steps
     constexpr bool TAIL16 = (D % 32) != 0;      // one more step, upper k half zero
@@ -181,20 +201,30 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
     constexpr int NVL = (DEC_CHUNK * LPR + 63) / 64;   // pieces of the value tile per lane
     constexpr int VS = D + 16;                  // value tile row stride in LDS (elements): rows shift by 8 banks
 
-    __shared__ __attribute__((aligned(16))) uint16_t v_s[DEC_CHUNK * VS];
+    constexpr int REGION = dec_region_bytes(D);
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int wv = threadIdx.x >> 6;             // wave of the workgroup
+    uint16_t* v_s = reinterpret_cast<uint16_t*>(lds_raw + (size_t)wv * REGION);
+    [[maybe_unused]] uint16_t* new_s =           // FUSED: the new token's k and v, behind the waves' regions
+        reinterpret_cast<uint16_t*>(lds_raw + (size_t)merge_waves * REGION + (size_t)wv * 4 * D);
 
     // blockIdx.y: kv head and, when more than 16 query heads share it, which 16 of them
     const int group = Hq / Hkv, blocks = (group + DEC_MAX_GROUP - 1) / DEC_MAX_GROUP;
-    const int di = blockIdx.x, kvh = blockIdx.y / blocks, hb = blockIdx.y - kvh * blocks, sp = blockIdx.z;
+    const int di = blockIdx.x, kvh = blockIdx.y / blocks, hb = blockIdx.y - kvh * blocks;
+    const int sp = merge_waves > 1 ? wv : (int)blockIdx.z;
     const int seg = seg_ids ? seg_ids[di] : di;
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int h0 = kvh * group + hb * DEC_MAX_GROUP;             // first query head of this wave
     const int G = min(DEC_MAX_GROUP, group - hb * DEC_MAX_GROUP);  // and how many it has
     const int t = cu_q[seg];
     const int pos_q = q_start[seg];
     const int start = kv_start[seg];
+    // A merging workgroup cuts its own request into merge_waves even splits (counted from
+    // position 0), whatever the longest request of the step is.
+    if (merge_waves > 1) split_tokens = max(1, (pos_q + DEC_CHUNK * merge_waves) / (DEC_CHUNK * merge_waves)) * DEC_CHUNK;
     const DecodeRange rg = decode_range(pos_q, start, window, split_tokens, sp);
-    if (rg.lo > rg.hi) return;
+    const bool empty = rg.lo > rg.hi;            // a split beyond the request's keys
+    if (empty && merge_waves == 1) return;       // (in a merging workgroup the wave stays for the barrier, with no keys)
     const int* pt = page_table + cu_pages[seg];
     const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
 
@@ -204,7 +234,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
     bf16x8_t bq_tail = z8;
     // FUSED: the new token is not among the keys of the passes; its key and value come from the
     // projection and are added at the end
-    [[maybe_unused]] const bool has_new = FUSED && rg.hi == pos_q;
+    [[maybe_unused]] const bool has_new = FUSED && !empty && rg.hi == pos_q;
     const int key_hi = has_new ? pos_q - 1 : rg.hi;          // last key position read from the cache
     const int c_begin = (rg.lo / DEC_CHUNK) * DEC_CHUNK;
     // row in the pools of this lane's key of the pass that starts at c (clamped into the split so
@@ -216,7 +246,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
         return pt[pi] * P + (idx - pi * P);
     };
     int row_next = 0;
-    [[maybe_unused]] __shared__ __attribute__((aligned(16))) uint16_t new_s[FUSED ? 2 * D : 8];   // the new token's k, v
     if constexpr (FUSED) {
         static_assert(!TAIL16 && D32 % 2 == 0, "the fused preparation needs a head size that is a multiple of 64");
         const size_t width = (size_t)(Hq + 2 * Hkv) * D;
@@ -302,7 +331,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
             const int r = __shfl(row, e / LPR, 64);
             vv[i] = *reinterpret_cast<const uint4_t*>(v_pool + ((size_t)r * Hkv + kvh) * D + (e % LPR) * 8);
         }
-        __syncthreads();                           // the previous pass has read its value tile
+        WAVE_SYNC();                               // the previous pass has read its value tile
 #pragma unroll
         for (int i = 0; i < NVL; ++i) {
             const int e = min(lane + 64 * i, DEC_CHUNK * LPR - 1);
@@ -357,7 +386,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
             }
         }
         m_run = m_new;
-        __syncthreads();                           // the value tile is complete in LDS
+        WAVE_SYNC();                               // the value tile is complete in LDS
 
         // ---- O^T += V^T P^T, 32 keys per MFMA
 #pragma unroll
@@ -383,7 +412,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
             // ---- the new token as one more key: its score by plain 32-bit sums of bf16 products
             // (this lane's 8*D32 elements, then over the four lanes of the head), then the same
             // running maximum and sums as in a pass
-            __syncthreads();
+            WAVE_SYNC();
             float dot = 0.f;
 #pragma unroll
             for (int j = 0; j < D32; ++j) {
@@ -413,6 +442,42 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
         }
     }
 
+    if (merge_waves > 1) {
+        // ---- this wave's sums into its own region (its value tile is no longer needed), then
+        // every thread of the workgroup merges a piece of the result over the waves, in wave order
+        WAVE_SYNC();
+        float* mine = reinterpret_cast<float*>(lds_raw + (size_t)wv * REGION);      // [16][D] sums, then [16][2] m, l
+#pragma unroll
+        for (int dt = 0; dt < D16; ++dt) *reinterpret_cast<float4_t*>(mine + n * D + dt * 16 + 4 * g) = acc[dt];
+        if (g == 0) {
+            mine[16 * D + 2 * n] = m_run;
+            mine[16 * D + 2 * n + 1] = l_run;
+        }
+        __syncthreads();
+        const int threads = merge_waves * 64;
+        for (int idx = threadIdx.x; idx < G * (D / 4); idx += threads) {
+            const int hn = idx / (D / 4), d4 = idx - hn * (D / 4);
+            float mx = -INFINITY;
+            for (int w = 0; w < merge_waves; ++w)
+                mx = fmaxf(mx, reinterpret_cast<const float*>(lds_raw + (size_t)w * REGION)[16 * D + 2 * hn]);
+            float4_t o = {0.f, 0.f, 0.f, 0.f};
+            float l = 0.f;
+            for (int w = 0; w < merge_waves; ++w) {
+                const float* other = reinterpret_cast<const float*>(lds_raw + (size_t)w * REGION);
+                const float mw = other[16 * D + 2 * hn];
+                const float e = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - mx);
+                const float4_t a = *reinterpret_cast<const float4_t*>(other + hn * D + 4 * d4);
+                o[0] = fmaf(a[0], e, o[0]); o[1] = fmaf(a[1], e, o[1]);
+                o[2] = fmaf(a[2], e, o[2]); o[3] = fmaf(a[3], e, o[3]);
+                l += other[16 * D + 2 * hn + 1] * e;
+            }
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            const uint2 packed = {pack2(o[0] * inv, o[1] * inv), pack2(o[2] * inv, o[3] * inv)};
+            *reinterpret_cast<uint2*>(out + ((size_t)t * Hq + h0 + hn) * D + 4 * d4) = packed;
+        }
+        return;
+    }
+
     // ---- partial results of this split: lane (n, g) holds head n, columns 16dt + 4g .. +3
     if (n < G) {
         float* pa = part_acc + (((size_t)di * Hq + h0 + n) * max_splits + sp) * D;
@@ -429,29 +494,47 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2
 #define DEC_CAT2(a, b) a##b
 #define DEC_CAT(a, b) DEC_CAT2(a, b)
 // head sizes 16*(4*DEC_PART+1) .. 16*(4*DEC_PART+4)
+template <int N, bool FUSED>
+static int dec_launch_one(dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm, const bf16* kp,
+                          const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq,
+                          const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,
+                          int split_tokens, int max_splits, DecodeFused fz, int merge_waves, bf16* out) {
+    constexpr int D = 16 * N;
+    const size_t lds = (size_t)merge_waves * (dec_region_bytes(D) + (FUSED ? 4 * D : 0));
+    auto kern = attn_decode_kernel<N, FUSED>;
+    static size_t allowed = 64 * 1024;                        // per instantiation: raised when needed
+    if (lds > allowed) {
+        if (lds > 160 * 1024 ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+            return RA_ERR_ARG;
+        allowed = lds;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(64 * merge_waves), lds, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs,
+                       segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz, merge_waves, out);
+    return RA_OK;
+}
+
 extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t st, const bf16* q, float* pa,
                                               float* pm, const bf16* kp, const bf16* vp, const int* pt,
                                               const int* cup, const int* kvs, const int* cuq,
                                               const int* qs, const int* segs, int Hq, int Hkv, int P,
                                               float scale, int window, int split_tokens,
-                                              int max_splits, DecodeFused fz) {
+                                              int max_splits, DecodeFused fz, int merge_waves, bf16* out) {
+#define DEC_ARGS grid, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, \
+                 split_tokens, max_splits, fz, merge_waves, out
     if (fz.qkv != nullptr) {                      // head sizes 64, 128, 192, 256: one of them in each part
         if (D16 != 4 * DEC_PART + 4) return RA_ERR_ARG;
-        hipLaunchKernelGGL((attn_decode_kernel<4 * DEC_PART + 4, true>), grid, dim3(64), 0, st, q, pa, pm, kp, vp,
-                           pt, cup, kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz);
-        return RA_OK;
+        return dec_launch_one<4 * DEC_PART + 4, true>(DEC_ARGS);
     }
-#define DEC_CASE(N)                                                                                \
-    case N:                                                                                        \
-        hipLaunchKernelGGL((attn_decode_kernel<N, false>), grid, dim3(64), 0, st, q, pa, pm, kp, vp, pt, cup, \
-                           kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz); \
-        return RA_OK;
     switch (D16) {
-        DEC_CASE(4 * DEC_PART + 1) DEC_CASE(4 * DEC_PART + 2) DEC_CASE(4 * DEC_PART + 3)
-        DEC_CASE(4 * DEC_PART + 4)
+        case 4 * DEC_PART + 1: return dec_launch_one<4 * DEC_PART + 1, false>(DEC_ARGS);
+        case 4 * DEC_PART + 2: return dec_launch_one<4 * DEC_PART + 2, false>(DEC_ARGS);
+        case 4 * DEC_PART + 3: return dec_launch_one<4 * DEC_PART + 3, false>(DEC_ARGS);
+        case 4 * DEC_PART + 4: return dec_launch_one<4 * DEC_PART + 4, false>(DEC_ARGS);
         default: return RA_ERR_ARG;
     }
-#undef DEC_CASE
+#undef DEC_ARGS
 }
 #endif  // DEC_PART
 
@@ -460,7 +543,7 @@ extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t s
 #define DEC_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm,        \
     const bf16* kp, const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq,   \
     const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,                 \
-    int split_tokens, int max_splits, DecodeFused fz
+    int split_tokens, int max_splits, DecodeFused fz, int merge_waves, bf16* out
 extern "C" int ra_dec_part_0(DEC_PART_ARGS);
 extern "C" int ra_dec_part_1(DEC_PART_ARGS);
 extern "C" int ra_dec_part_2(DEC_PART_ARGS);
@@ -504,22 +587,37 @@ __global__ __launch_bounds__(128) void attn_decode_combine_kernel(
 // part_acc: fp32 [n_dec, Hq, max_splits, D]; part_ml: fp32 [n_dec, Hq, max_splits, 2].
 // max_splits is the number of splits of the request with the most; requests with fewer leave
 // the rest untouched and the merge does not read it.
+// merge != 0: the splits of a request are the waves of one workgroup and are merged there (no partial
+// sums in memory, no merge kernel); max_splits must not exceed ra_attention_decode_merge_waves(D).
+// Most waves (splits) of a merging workgroup for head size D: what the LDS holds and the kernel's
+// launch bounds allow.
+extern "C" int ra_attention_decode_merge_waves(int D) {
+    if (D % 16 != 0 || D < 16 || D > 256) return 0;
+    const int region = (DEC_CHUNK * (D + 16) * 2 > 16 * (D + 2) * 4) ? DEC_CHUNK * (D + 16) * 2 : 16 * (D + 2) * 4;
+    const int by_lds = (160 * 1024 - 1024) / (region + 4 * D);
+    const int by_bounds = D <= 128 ? 8 : 4;
+    return by_lds < by_bounds ? by_lds : by_bounds;
+}
+
 static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const bf16* kp, const bf16* vp,
                          const int* page_table, const int* cu_pages, const int* kv_start, const int* cu_q,
                          const int* q_start, const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
                          float scale, int window, int split_tokens, int max_splits, DecodeFused fz,
-                         hipStream_t st) {
+                         int merge, hipStream_t st) {
     if (n_dec <= 0) return RA_OK;
     if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 ||
         split_tokens <= 0 || split_tokens % DEC_CHUNK != 0 || max_splits <= 0 || max_splits > 65535 || P <= 0)
         return RA_ERR_ARG;
     const int head_blocks = Hkv * ((Hq / Hkv + DEC_MAX_GROUP - 1) / DEC_MAX_GROUP);
     if (head_blocks > 65535) return RA_ERR_ARG;
-    dim3 grid(n_dec, head_blocks, max_splits);
+    if (merge && (max_splits < 2 || max_splits > ra_attention_decode_merge_waves(D) || window > 0)) return RA_ERR_ARG;
+    dim3 grid(n_dec, head_blocks, merge ? 1 : max_splits);
+    const int merge_waves = merge ? max_splits : 1;
     int rc;
     const int d16 = D / 16;
 #define DEC_GO(N) rc = ra_dec_part_##N(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, \
-                                       q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz)
+                                       q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz, \
+                                       merge_waves, (bf16*)out)
     switch ((d16 - 1) / 4) {
         case 0: DEC_GO(0); break;
         case 1: DEC_GO(1); break;
@@ -530,6 +628,7 @@ static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const 
 #undef DEC_GO
     if (rc != RA_OK) return rc;
     if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
+    if (merge) return RA_OK;
     hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128),
                        (size_t)max_splits * sizeof(float), st, pa, pm, (bf16*)out, kv_start, cu_q,
                        q_start, seg_ids, Hq, D, window, split_tokens, max_splits);
@@ -542,11 +641,11 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
                                         const int* kv_start, const int* cu_q, const int* q_start,
                                         const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
                                         float scale, int window, int split_tokens, int max_splits,
-                                        void* stream) {
+                                        int merge, void* stream) {
     DecodeFused none = {};
     return decode_launch((const bf16*)q, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
-                         Hkv, D, P, scale, window, split_tokens, max_splits, none, (hipStream_t)stream);
+                         Hkv, D, P, scale, window, split_tokens, max_splits, none, merge, (hipStream_t)stream);
 }
 
 // The same for requests whose new token has not been prepared: qkv [tokens, (Hq + 2 Hkv) D] as the
@@ -560,13 +659,13 @@ extern "C" int ra_attention_decode_fused_bf16(const void* qkv, void* out, void* 
                                               int Hkv, int D, int P, float scale, int window,
                                               int split_tokens, int max_splits, const float* w_q,
                                               const float* w_k, float eps, const float* cos_t,
-                                              const float* sin_t, void* stream) {
+                                              const float* sin_t, int merge, void* stream) {
     if (qkv == nullptr || D % 64 != 0 || (w_q == nullptr) != (w_k == nullptr) ||
         (cos_t == nullptr) != (sin_t == nullptr))
         return RA_ERR_ARG;
     DecodeFused fz = {(const bf16*)qkv, w_q, w_k, eps, cos_t, sin_t, (bf16*)k_pool, (bf16*)v_pool};
     return decode_launch(nullptr, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
-                         Hkv, D, P, scale, window, split_tokens, max_splits, fz, (hipStream_t)stream);
+                         Hkv, D, P, scale, window, split_tokens, max_splits, fz, merge, (hipStream_t)stream);
 }
 #endif  // DEC_API
