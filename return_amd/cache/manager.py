@@ -147,6 +147,25 @@ class CacheManager:
         self._step_requests: List = []
         self.version = 0            # changes whenever any request's page list changes
 
+    @staticmethod
+    def pool_bytes(cache_layers: Dict[int, object], page_size: int, max_token: int, max_requests: int,
+                   dtype: torch.dtype) -> int:
+        """Bytes of device memory that a manager with these arguments allocates (pools with their
+        spare page, state with its spare slot)."""
+        item = torch.empty((), dtype=dtype).element_size()
+        pages = int(max_token) // int(page_size) + 1
+        total = 0
+        for spec in cache_layers.values():
+            if isinstance(spec, PagedKVSpec):
+                total += 2 * pages * int(page_size) * spec.num_kv_heads * spec.head_dim * item
+            elif isinstance(spec, StateSpec):
+                for _, shape, dt in spec.tensors:
+                    n = 1
+                    for d in shape:
+                        n *= int(d)
+                    total += (int(max_requests) + 1) * n * torch.empty((), dtype=_DTYPES[dt]).element_size()
+        return total
+
     # ------------------------------------------------------------------ requests
     def add_request(self, rid) -> int:
         if rid in self.live:

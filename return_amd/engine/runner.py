@@ -58,6 +58,7 @@ class ModelRunner:
         del weights
         if ec.tune_products and self.rt.dtype == torch.bfloat16 and hasattr(self.rt.ops, "tune_products"):
             self.rt.ops.tune_products(self.rt.products, max_rows=ec.max_reside)
+        self._check_cache_fits()
         self.cache = CacheManager(self.model.cache_layers(), ec.page_size, ec.max_token,
                                   ec.max_reside, self.rt.dtype, self.rt.device)
         self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device)
@@ -85,6 +86,22 @@ class ModelRunner:
         self._feed_at_dev = torch.zeros(n, dtype=torch.int64, device=self.rt.device)
         self._launches = 0
         self._last_picked: Optional[torch.Tensor] = None
+
+    def _check_cache_fits(self) -> None:
+        """One clear error, before anything is allocated, when the cache asked for cannot fit beside the weights."""
+        if self.rt.device.type != "cuda":
+            return
+        ec = self.engine_config
+        layers = self.model.cache_layers()
+        need = CacheManager.pool_bytes(layers, ec.page_size, ec.max_token, ec.max_reside, self.rt.dtype)
+        torch.cuda.empty_cache()
+        free, _ = torch.cuda.mem_get_info(self.rt.device)
+        if need > free:
+            per_token = CacheManager.pool_bytes(layers, 1, 1, 0, self.rt.dtype) // 2 or 1
+            fits = max(0, free // per_token // ec.page_size - 1) * ec.page_size
+            raise ValueError(
+                f"the cache for max_token={ec.max_token} takes {need / 2 ** 30:.1f} GiB, but {free / 2 ** 30:.1f} GiB "
+                f"of device memory are free beside the weights: about max_token={fits} would fit")
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request_id) -> None:

@@ -223,3 +223,13 @@ def test_pad_tables_adds_rows_on_the_spare_page_only():
     assert cm.state[2]["s"].shape[0] == 4
     cm.end_step()
     cm.check_invariants()
+
+
+def test_pool_bytes_is_what_the_manager_allocates():
+    layers = {0: PagedKVSpec(2, 8, None), 1: PagedKVSpec(2, 8, None), 2: PagedKVSpec(1, 24, 5),
+              3: StateSpec((("conv", (3, 2), "bfloat16"), ("rec", (2, 4, 4), "float32")))}
+    for dtype in (torch.bfloat16, torch.float32):
+        cm = CacheManager(layers, page_size=4, max_token=50, max_requests=3, dtype=dtype)
+        held = sum(g.pool.numel() * g.pool.element_size() for g in cm.groups)
+        held += sum(t.numel() * t.element_size() for ts in cm.state.values() for t in ts.values())
+        assert CacheManager.pool_bytes(layers, 4, 50, 3, dtype) == held

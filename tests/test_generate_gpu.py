@@ -156,6 +156,12 @@ def test_command_line_turns_of_a_session(folder_a, tmp_path):
     assert stats["resident"] == 0 and stats["kv_used"] == [0]
 
 
+def test_a_cache_that_cannot_fit_is_refused_before_it_is_allocated(folder_a):
+    from return_amd.engine import Engine
+    with pytest.raises(ValueError, match=r"max_token=1073741824 takes .* GiB.*would fit"):
+        Engine(folder_a, dtype="float32", page_size=16, max_token=2 ** 30, max_reside=2)
+
+
 def test_the_library_is_the_one_that_runs():
     """The HIP library is loaded in this process; there is nothing else behind the kernels."""
     from return_amd.kernels.hip_ops import HipOps
