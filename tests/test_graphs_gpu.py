@@ -49,19 +49,23 @@ def test_graph_replays_match_eager(folder_b, dtype):
     assert te == tg and torch.equal(logits_e, logits_g)
 
 
-@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32", "bfloat16, splits merged in the workgroup"])
 def test_batch_filled_up_to_a_graph_size(folder_b, dtype):
     """Eleven requests run from the graph of sixteen: the five added rows write and read the
     spare page only; logits, tokens and every page that a request holds equal the eager run.
     (Products by rule: a measured plan may form products of 11 and of 16 rows in different ways,
-    which differ in rounding.)"""
+    which differ in rounding.) Once more with the decode attention that merges a request's splits
+    inside one workgroup, where the added rows are workgroups with a single key."""
     V = TINY_B["vocab_size"]
     lens = [5, 17, 33, 64, 2, 90, 16, 47, 1, 129, 31]
+    dtype, _, merged = dtype.partition(",")
 
     def make(use_graphs):
         ec = EngineConfig(dtype=dtype, page_size=16, max_token=4096, max_reside=16, max_step_tokens=512,
                           prefill_chunk=512, use_graphs=use_graphs, tune_products=False)
         r = ModelRunner(folder_b, engine_config=ec)
+        if merged:
+            r.rt.ops.decode_merge_round = 1          # every count of requests is a whole round
         for i, n in enumerate(lens):
             r.add_request(i)
             r.step([StepEntry(i, tt.random_tokens(V, n, seed=100 + n), [])])

@@ -69,6 +69,24 @@ def test_replay_matches_plain(model, dtype, cut):
     assert all(g.pages.in_use() == 0 for g in runner.cache.groups)
 
 
+@pytest.mark.parametrize("cut", ["tail_decoded", "mixed"])
+def test_decode_attention_that_merges_inside_the_workgroup(model, cut):
+    """The decode attention merges a request's splits inside one workgroup when the (request, kv
+    head) pairs make whole rounds over the CUs, which tiny models never do: here every count is a
+    whole round, so that each decoded token of the traces takes that path (requests of every length
+    from one token on, beside each other, on pages used again)."""
+    folder, raw, reqs, want = model
+    steps = {"tail_decoded": tt.tail_decoded, "mixed": tt.mixed}[cut](reqs)
+    runner = make_runner(folder, "bfloat16", tt.peak_tokens(steps))
+    ops = runner.rt.ops
+    ops.decode_merge_round = 1
+    seen = []
+    splits = ops._decode_splits
+    ops._decode_splits = lambda *a, **k: (seen.append(splits(*a, **k)) or seen[-1])
+    compare(tt.run_in_process(runner, steps), want, reqs, "bfloat16")
+    assert any(merge for _, _, merge in seen), "no step took the merging path"
+
+
 @pytest.mark.parametrize("page", [8, 32, 64])
 def test_other_page_sizes(folder_b, page):
     reqs = requests_for(TINY_B["vocab_size"], TINY_B["max_position_embeddings"])
