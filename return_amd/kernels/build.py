@@ -124,8 +124,9 @@ def build(force: bool = True) -> str:
             return have
     hipcc = _hipcc()
     out_dir = _writable_dir()
-    obj_dir = os.path.join(out_dir, "_build")
-    os.makedirs(obj_dir, exist_ok=True)
+    # objects in a folder of this process's own: two processes that build at once (two first
+    # calls in a fresh checkout) do not write, link or delete each other's files
+    obj_dir = tempfile.mkdtemp(prefix="_build-", dir=out_dir)
     units = compile_units()
     t0 = time.time()
     _say(f"compiling {len(units)} HIP units for {ARCH} into {out_dir}")
@@ -146,15 +147,16 @@ def build(force: bool = True) -> str:
         workers = min(len(units), max(1, min(8, os.cpu_count() or 1)))
         with concurrent.futures.ThreadPoolExecutor(workers) as pool:
             objs = list(pool.map(one, units))
-        tmp = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
+        tmp = os.path.join(out_dir, f".{LIB_NAME}.{os.path.basename(obj_dir)}")
         _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], "linking")
         lib = os.path.join(out_dir, LIB_NAME)
         os.replace(tmp, lib)
-        with open(lib + ".hash", "w") as f:
+        with open(tmp + ".hash", "w") as f:
             f.write(source_hash())
+        os.replace(tmp + ".hash", lib + ".hash")
     finally:
         done.set()
-    shutil.rmtree(obj_dir, ignore_errors=True)
+        shutil.rmtree(obj_dir, ignore_errors=True)
     _say(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
 
