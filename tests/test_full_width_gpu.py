@@ -95,3 +95,40 @@ def test_full_width_generation_through_graphs(wide):
             if tok != int(top2.indices[0]):           # a near tie that bfloat16 may decide the other way
                 assert float(top2.values[0] - top2.values[1]) < 0.1
             assert abs(r.output_logprobs[i] - plain.chosen_logprob(rows[i], tok)) < 0.1
+
+
+def test_full_width_graph_replays_equal_the_eager_steps(wide):
+    """Twelve requests decode from the graph of sixteen at full width, where the products of a step
+    are the library's: every replay gives the bits of the eager step, with eager work of the
+    program's own (another request's prompt) and synchronisations between the replays."""
+    from return_amd.config import EngineConfig
+    from return_amd.engine import ModelRunner, StepEntry
+    folder, _, _ = wide
+    V = WIDE["vocab_size"]
+    lens = [5, 17, 300, 64, 2, 90, 16, 47, 1, 129, 31, 200]
+
+    def make(use_graphs):
+        ec = EngineConfig(dtype="bfloat16", page_size=16, max_token=8192, max_reside=16, max_step_tokens=1024,
+                          prefill_chunk=1024, use_graphs=use_graphs, tune_products=False)
+        r = ModelRunner(folder, engine_config=ec)
+        for i, n in enumerate(lens):
+            r.add_request(i)
+            r.step([StepEntry(i, tt.random_tokens(V, n, seed=300 + n), [])])
+        return r
+
+    eager, graph = make(False), make(True)
+    ids = list(range(len(lens)))
+    toks = [3 + i for i in ids]
+    zeros, ones = [0.0] * len(ids), [1.0] * len(ids)
+    for step in range(24):
+        te, le, logits_e = eager.decode_and_sample(ids, toks, zeros, [0] * len(ids), ones, zeros)
+        tg, lg, logits_g = graph.decode_and_sample(ids, toks, zeros, [0] * len(ids), ones, zeros)
+        assert torch.equal(logits_e, logits_g), f"replay {step} differs from the eager step"
+        assert te == tg and le == lg
+        toks = te
+        if step % 5 == 0:
+            graph.add_request("x")
+            graph.step([StepEntry("x", tt.random_tokens(V, 40, seed=step), [39])])
+            graph.free_request("x")
+            torch.cuda.synchronize()
+    assert {k[0] for k in graph._graphs} == {16}
