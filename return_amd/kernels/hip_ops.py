@@ -64,6 +64,8 @@ def _declare(lib):
         "ra_gemm_mfma_bf16": [P, P, P, I, I, I, I, P],
         "ra_gemm_resident_bf16": [P, P, P, I, I, I, I, I, I, P],
         "ra_gemm_resident_fits": [I, I, I],
+        "ra_gemm_sweep_bf16": [P, P, P, I, I, I, I, I, I, P],
+        "ra_gemm_sweep_fits": [I, I],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, I, P],
@@ -101,7 +103,8 @@ class HipOps:
         self.decode_split_tokens = 0         # keys per split of the decode attention; 0: by batch size
         # a request's splits as one workgroup that merges them itself: one such workgroup fills a CU
         # (LDS), so it pays when the (request, kv head) pairs come to whole rounds over the CUs
-        self.decode_merge_round = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self.cu_count = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self.decode_merge_round = self.cu_count
         self.prefill_key_split = 0           # groups of waves that share a q tile's keys (1 or 2); 0: by the number of tiles
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
@@ -131,6 +134,17 @@ class HipOps:
         if out_dtype == torch.float32:
             return M <= 16                   # more rows: the library, or the tiled MFMA product
         return M <= 4 or (M <= 16 and N * K <= (32 << 20)) or (M <= 32 and N * K <= (16 << 20))
+
+    def use_sweep(self, M, N, K, gated):
+        """Whether the product that reads W as one sweep through memory (one workgroup per CU, column
+        c with workgroup c % CUs) is the rule's choice for x [M, K] and N result columns. Measured on
+        MI355X at 1 to 16 rows: 12 against 15 µs (q/k/v of the 8B shape), 10 against 11 (o), 36 against
+        41 (gate-up) for the x-resident and skinny products; on the output head's 152 thousand rows
+        the x-resident product is ahead (two workgroups per CU hide each other's tile ends)."""
+        if not self.lib.ra_gemm_sweep_fits(M, K):
+            return False
+        rows = N * (2 if gated else 1)
+        return 8 * self.cu_count <= rows <= 128 * self.cu_count
 
     def use_resident(self, M, N, K, gated):
         """Whether the product with x resident in LDS beats the skinny product for x [M, K] and
@@ -315,6 +329,8 @@ class HipOps:
         hit = self.product_plan.get((self._rows_step(M), N, K, False, out_dtype))
         if hit is not None:
             return hit
+        if out_dtype in (torch.bfloat16, torch.float32) and self.use_sweep(M, N, K, False):
+            return "sweep"
         if out_dtype in (torch.bfloat16, torch.float32) and self.use_resident(M, N, K, False):
             return "resident512" if M <= 8 else "resident256"
         if self.use_skinny(M, N, K, out_dtype):
@@ -327,6 +343,8 @@ class HipOps:
         hit = self.product_plan.get((self._rows_step(M), I, K, True, torch.bfloat16))
         if hit is not None:
             return hit
+        if self.use_sweep(M, I, K, True):
+            return "sweep"
         if self.use_resident(M, I, K, True):
             return "resident512" if M <= 8 else "resident256"
         if 0 < M <= self.gated_skinny_rows and K % 8 == 0:
@@ -341,7 +359,10 @@ class HipOps:
                 return torch.matmul(x, w.t())          # library product, as the reference's F.linear
             return torch.mm(x, w.t(), out_dtype=torch.float32)   # bf16 operands, 32-bit sums and results
         y = torch.empty(M, N, dtype=out_dtype, device=self.device)
-        if how.startswith("resident"):
+        if how == "sweep":
+            self._check(self.lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, _code(out_dtype),
+                                                    self.cu_count, self._stream()), "gemm_sweep")
+        elif how.startswith("resident"):
             self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, 0, _code(out_dtype),
                                                        int(how[8:]), self._stream()), "gemm_resident")
         elif how == "skinny":
@@ -375,7 +396,10 @@ class HipOps:
         M, K = x.shape
         I = w_gate_up.shape[0] // 2
         out = torch.empty(M, I, dtype=x.dtype, device=self.device)
-        if how.startswith("resident"):
+        if how == "sweep":
+            self._check(self.lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K, 1, _code(x.dtype),
+                                                    self.cu_count, self._stream()), "gemm_sweep_gated")
+        elif how.startswith("resident"):
             self._check(self.lib.ra_gemm_resident_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), M, I, K, 1,
                                                        _code(x.dtype), int(how[8:]), self._stream()),
                         "gemm_resident_gated")
@@ -409,6 +433,8 @@ class HipOps:
                 c.append("skinny")
         if self.lib.ra_gemm_resident_fits(M, K, 1 if gated else 0):
             c += ["resident256", "resident512"]
+        if self.lib.ra_gemm_sweep_fits(M, K):
+            c.append("sweep")
         return c
 
     def tune_products(self, products, max_rows=64, margin=0.93):

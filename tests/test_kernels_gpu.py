@@ -222,6 +222,38 @@ def test_resident_product(ops, ref, M, N, K, grid):
     assert not ops.lib.ra_gemm_resident_fits(16, 8192, 0) and ops.lib.ra_gemm_resident_fits(8, 8192, 0)
 
 
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("N,K", [(6144, 4096), (2500, 2560), (700, 4096), (4099, 520), (37, 64)])
+def test_product_that_sweeps_the_weight(ops, N, K, gated):
+    """The product that reads W as one sweep (column c with workgroup c % CUs): widths that fill
+    every wave's 512 columns and widths that leave waves idle, column counts that are no multiple of
+    the workgroups or of a tile, fewer columns than workgroups, 1 to 16 rows, both result types, the
+    gated form; and what it does not take is refused."""
+    from return_amd.kernels.hip_ops import _code, _ptr
+    lib, st = ops.lib, torch.cuda.current_stream().cuda_stream
+    w = rnd((2 if gated else 1) * N, K, dtype=torch.bfloat16, seed=N, scale=0.05)
+    for M in (1, 2, 5, 8, 13, 16):
+        x = rnd(M, K, dtype=torch.bfloat16, seed=M + 1)
+        want = x.double() @ w.double().t()
+        if gated:
+            g, u = want[:, :N], want[:, N:]
+            want = g * torch.sigmoid(g) * u
+        for out_dtype in ((torch.bfloat16,) if gated else (torch.bfloat16, torch.float32)):
+            for grid in (ops.cu_count, 7):
+                y = torch.full((M, N), 9.0, dtype=out_dtype, device=DEV)
+                assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(gated), _code(out_dtype), grid, st) == 0
+                if out_dtype == torch.float32:
+                    torch.testing.assert_close(y.double(), want, atol=1e-4 * K ** 0.5, rtol=1e-5)
+                else:
+                    torch.testing.assert_close(y.float(), want.float(), **tol(torch.bfloat16))
+    y = torch.empty(17, N, dtype=torch.bfloat16, device=DEV)
+    x = rnd(17, K, dtype=torch.bfloat16)
+    assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), 17, N, K, int(gated), _code(torch.bfloat16), 256, st) != 0
+    assert not lib.ra_gemm_sweep_fits(8, 4104) and not lib.ra_gemm_sweep_fits(8, 4100) and lib.ra_gemm_sweep_fits(16, 4096)
+    if gated:
+        assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), 8, N, K, 1, _code(torch.float32), 256, st) != 0
+
+
 @pytest.mark.parametrize("N,K", [(331, 120), (1000, 264), (48, 4096)])
 def test_every_way_to_form_a_product(ops, monkeypatch, N, K):
     """linear and linear_silu_mul under every way the plan may name, at every measured row count:
@@ -252,7 +284,8 @@ def test_every_way_to_form_a_product(ops, monkeypatch, N, K):
             y = ops.linear_silu_mul(x, w)
             torch.testing.assert_close(y.float(), (g * torch.sigmoid(g) * u).float(), **tol(torch.bfloat16))
             ways.add("gated " + how)
-    assert {"library", "skinny", "resident256", "resident512", "gated two", "gated skinny", "gated resident512"} <= ways
+    assert {"library", "skinny", "resident256", "resident512", "sweep", "gated two", "gated skinny",
+            "gated resident512", "gated sweep"} <= ways
 
 
 def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
@@ -282,11 +315,11 @@ def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
     assert not calls and plan == before
     # a way that is clearly faster replaces the rule's, one that is barely faster does not
     cands = ops._candidates(1, 768, 256, False, torch.bfloat16)
-    assert cands == ["library", "skinny", "resident256", "resident512"]
+    assert cands == ["library", "skinny", "resident256", "resident512", "sweep"]
     plan.clear()
     assert ops.route_linear(1, 768, 256, torch.bfloat16) == "skinny"            # the rule
     key = (1, 768, 256, False, torch.bfloat16)
-    for seconds, choice in (([1.0, 0.95, 0.5, 0.96], "resident256"), ([0.9, 0.95, 1.0, 0.96], None)):
+    for seconds, choice in (([1.0, 0.95, 0.5, 0.96, 0.97], "resident256"), ([0.9, 0.95, 1.0, 0.96, 0.97], None)):
         it = iter(seconds)
         monkeypatch.setattr(ops, "_time_over", lambda *a: next(it))
         plan.clear(); measured.clear()
