@@ -1,5 +1,5 @@
-// y = x @ W^T for up to 16 rows of x and K up to 4,096, with W read as one sweep through memory: the
-// decode-time product of a small batch, which is bound by reading W once.
+// y = x @ W^T for up to 16 rows of x with W read as one sweep through memory: the decode-time
+// product of a small batch, which is bound by reading W once.
 // Layout as in the reference's F.linear (rollout/monkey_patch/qwen3.py:21): x [M, K], W [N, K],
 // y [M, N].
 //
@@ -16,6 +16,9 @@
 // Results: bfloat16 or fp32 [M, N]; GATED (W = [Wg; Wu], rollout/monkey_patch/qwen3.py:103): a tile
 // is 8 gate rows and the 8 up rows of the same columns, the result silu(g) * u as [M, N]
 // (rollout/fused.py:103-114).
+// K beyond the 4,096 columns that eight waves cover at once (gemm_sweep_long_kernel): a tile's rows
+// are taken in spans of 4,096 columns, one after the other, each with its own B operands (read again
+// for every tile; they come from L2).
 // Needs K % 8 == 0.
 #include "common.h"
 
@@ -110,14 +113,103 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
     }
 }
 
+
+#define SW_SPAN (SW_WAVES * SW_KW)        // columns of K that the eight waves cover at once
+
+template <bool GATED, typename TO>
+__global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
+    const bf16* __restrict__ x, const bf16* __restrict__ W, TO* __restrict__ out, int M, int N, int K) {
+    constexpr int COLS = GATED ? 8 : 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + (size_t)wave * 16 * SW_STRIDE;
+    float* red_both = reinterpret_cast<float*>(lds_raw + (size_t)SW_WAVES * 16 * SW_STRIDE * 2);
+    const int G = gridDim.x, b = blockIdx.x;
+    const int my_cols = N > b ? (N - 1 - b) / G + 1 : 0;
+    const int n_tiles = (my_cols + COLS - 1) / COLS;
+    if (n_tiles == 0) return;
+    const int spans = (K + SW_SPAN - 1) / SW_SPAN;
+    const int kb = wave * SW_KW;
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    bf16x8_t wreg[16];
+    auto fetch = [&](int t, int p) {
+        const int k = p * SW_SPAN + kb + lane * 8;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int col = b + G * (t * COLS + (GATED ? (i & 7) : i));
+            const size_t row = (GATED && i >= 8) ? (size_t)N + col : (size_t)col;
+            wreg[i] = (k < K && col < N) ? *reinterpret_cast<const bf16x8_t*>(W + row * K + k) : zero;
+        }
+    };
+    fetch(0, 0);
+
+    for (int t = 0; t < n_tiles; ++t) {
+        float4_t c = {0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < spans; ++p) {
+            bf16x8_t bx[SW_STEPS];                              // the span's columns of x as B operands
+#pragma unroll
+            for (int j = 0; j < SW_STEPS; ++j) {
+                const int k = p * SW_SPAN + kb + 32 * j + 8 * g;
+                bx[j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
+            }
+            SW_WAVE_SYNC();
+#pragma unroll
+            for (int i = 0; i < 16; ++i) *reinterpret_cast<bf16x8_t*>(&stage[i * SW_STRIDE + lane * 8]) = wreg[i];
+            if (p + 1 < spans) fetch(t, p + 1);
+            else if (t + 1 < n_tiles) fetch(t + 1, 0);
+            SW_WAVE_SYNC();
+#pragma unroll
+            for (int j = 0; j < SW_STEPS; ++j) {
+                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&stage[n * SW_STRIDE + 32 * j + 8 * g]);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bx[j], c, 0, 0, 0);
+            }
+        }
+        MFMA_SETTLE();
+        float* red = red_both + (t & 1) * (SW_WAVES * 16 * 17);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[(wave * 16 + 4 * g + i) * 17 + n] = c[i];
+        __syncthreads();
+        if (tid < 16 * COLS) {
+            const int mm = tid / COLS, r = tid % COLS;
+            const int col = b + G * (t * COLS + r);
+            if (mm < M && col < N) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < SW_WAVES; ++w) s += red[(w * 16 + r) * 17 + mm];
+                if constexpr (GATED) {
+                    float up = 0.f;
+#pragma unroll
+                    for (int w = 0; w < SW_WAVES; ++w) up += red[(w * 16 + 8 + r) * 17 + mm];
+                    s = s / (1.0f + expf(-s)) * up;
+                }
+                out[(size_t)mm * N + col] = from_f<TO>(s);
+            }
+        }
+    }
+}
+
 static size_t sweep_lds() { return (size_t)SW_WAVES * 16 * SW_STRIDE * 2 + (size_t)2 * SW_WAVES * 16 * 17 * 4; }
 
+// Whether the sweep takes x [M, K]: up to 16 rows, K in whole pieces of 8 up to 8 spans.
 extern "C" int ra_gemm_sweep_fits(int M, int K) {
-    return M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && K <= SW_WAVES * SW_KW;
+    return M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && K <= 8 * SW_SPAN;
 }
 
 template <bool GATED, typename TO>
 static int launch_sweep(int grid, hipStream_t st, const bf16* x, const bf16* W, TO* out, int M, int N, int K) {
+    if (K > SW_SPAN) {
+        auto long_kern = gemm_sweep_long_kernel<GATED, TO>;
+        static bool long_allowed = false;
+        if (!long_allowed) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(long_kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)sweep_lds()) != hipSuccess)
+                return RA_ERR_ARG;
+            long_allowed = true;
+        }
+        hipLaunchKernelGGL(long_kern, dim3(grid), dim3(SW_THREADS), sweep_lds(), st, x, W, out, M, N, K);
+        return RA_OK;
+    }
     auto kern = gemm_sweep_kernel<GATED, TO>;
     static bool allowed = false;                              // per instantiation: more than 64 KB of LDS
     if (!allowed) {

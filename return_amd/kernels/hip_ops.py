@@ -139,12 +139,15 @@ class HipOps:
         """Whether the product that reads W as one sweep through memory (one workgroup per CU, column
         c with workgroup c % CUs) is the rule's choice for x [M, K] and N result columns. Measured on
         MI355X at 1 to 16 rows: 12 against 15 µs (q/k/v of the 8B shape), 10 against 11 (o), 36 against
-        41 (gate-up) for the x-resident and skinny products; on the output head's 152 thousand rows
-        the x-resident product is ahead (two workgroups per CU hide each other's tile ends)."""
+        41 (gate-up), 100 against 118 (gate-up of the 32B shape, K = 5,120) for the x-resident and
+        skinny products; on the output head's 152 thousand rows the x-resident product is ahead (two
+        workgroups per CU hide each other's tile ends), and on few rows of many columns (down: one tile
+        a workgroup, K = 12,288) the library."""
         if not self.lib.ra_gemm_sweep_fits(M, K):
             return False
         rows = N * (2 if gated else 1)
-        return 8 * self.cu_count <= rows <= 128 * self.cu_count
+        least = 8 if K <= 4096 else 32                   # rows a workgroup, at least
+        return least * self.cu_count <= rows <= 256 * self.cu_count
 
     def use_resident(self, M, N, K, gated):
         """Whether the product with x resident in LDS beats the skinny product for x [M, K] and

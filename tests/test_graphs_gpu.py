@@ -119,8 +119,10 @@ def test_steps_launched_ahead_on_the_device(folder_b, dtype, use_graphs):
     news = [12, 1, 9, 2, 15, 7, 30, 4, 11, 26, 5]
 
     def run(lookahead, stops):
+        # products by rule: a request that is found finished a step late makes a batch of one row more,
+        # and a measured plan may form products of 8 and of 9 rows in ways that round differently
         eng = Engine(folder_b, dtype=dtype, page_size=16, max_token=4096, max_reside=11, max_step_tokens=128,
-                     prefill_chunk=64, use_graphs=use_graphs, lookahead=lookahead, seed=4)
+                     prefill_chunk=64, use_graphs=use_graphs, lookahead=lookahead, seed=4, tune_products=False)
         params = [SamplingParams(temperature=0.0 if i % 3 else 0.9, top_k=0 if i % 2 else 30, max_new_tokens=n,
                                  seed=i, stop_ids=stops if i == 6 else [])
                   for i, n in enumerate(news)]

@@ -223,10 +223,12 @@ def test_resident_product(ops, ref, M, N, K, grid):
 
 
 @pytest.mark.parametrize("gated", [False, True])
-@pytest.mark.parametrize("N,K", [(6144, 4096), (2500, 2560), (700, 4096), (4099, 520), (37, 64)])
+@pytest.mark.parametrize("N,K", [(6144, 4096), (2500, 2560), (700, 4096), (4099, 520), (37, 64), (4096, 12288), (300, 9728),
+                                 (5200, 4104)])
 def test_product_that_sweeps_the_weight(ops, N, K, gated):
     """The product that reads W as one sweep (column c with workgroup c % CUs): widths that fill
-    every wave's 512 columns and widths that leave waves idle, column counts that are no multiple of
+    every wave's 512 columns and widths that leave waves idle, widths of several spans of 4,096 (whole
+    ones and one that ends after 8 columns), column counts that are no multiple of
     the workgroups or of a tile, fewer columns than workgroups, 1 to 16 rows, both result types, the
     gated form; and what it does not take is refused."""
     from return_amd.kernels.hip_ops import _code, _ptr
@@ -249,7 +251,8 @@ def test_product_that_sweeps_the_weight(ops, N, K, gated):
     y = torch.empty(17, N, dtype=torch.bfloat16, device=DEV)
     x = rnd(17, K, dtype=torch.bfloat16)
     assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), 17, N, K, int(gated), _code(torch.bfloat16), 256, st) != 0
-    assert not lib.ra_gemm_sweep_fits(8, 4104) and not lib.ra_gemm_sweep_fits(8, 4100) and lib.ra_gemm_sweep_fits(16, 4096)
+    assert lib.ra_gemm_sweep_fits(8, 4104) and not lib.ra_gemm_sweep_fits(8, 4100) and lib.ra_gemm_sweep_fits(16, 32768)
+    assert not lib.ra_gemm_sweep_fits(8, 32776)
     if gated:
         assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), 8, N, K, 1, _code(torch.float32), 256, st) != 0
 
