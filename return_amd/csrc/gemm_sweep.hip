@@ -8,7 +8,8 @@
 // (measured here: such a sweep reads 201 MB in 31 µs; the same bytes as 16 rows x 512 B per wave,
 // the order of an MFMA operand read straight from memory, take 35 µs). Wave w has columns
 // 512w .. 512w+511 of K: a row of W is one load of 1 KB per wave, sixteen rows (a tile) are on their
-// way per lane while the tile before is multiplied. The tile goes through a part of LDS that is the
+// way per lane while the tile before is multiplied; a row of the next tile is asked for as soon as
+// the same row of this one has arrived, so the loads on their way never run out. The tile goes through a part of LDS that is the
 // wave's own (16 rows of 512 + 8 elements), from where it is read back as A operands of MFMA
 // 16x16x32 bf16 (lane (n, g): 16 bytes of row n at 32j + 8g); the wave's columns of x are B operands
 // that stay in registers for all tiles. The eight waves' partial tiles are added through LDS in wave
@@ -56,15 +57,13 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
 
     // row i of tile t: column b + G (COLS t + i % COLS), GATED: rows 8.. are the up rows
     bf16x8_t wreg[16];
-    auto fetch = [&](int t) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int col = b + G * (t * COLS + (GATED ? (i & 7) : i));
-            const size_t row = (GATED && i >= 8) ? (size_t)N + col : (size_t)col;
-            wreg[i] = (k_in && col < N) ? *reinterpret_cast<const bf16x8_t*>(W + row * K + kb + lane * 8) : zero;
-        }
+    auto fetch_row = [&](int t, int i) {
+        const int col = b + G * (t * COLS + (GATED ? (i & 7) : i));
+        const size_t row = (GATED && i >= 8) ? (size_t)N + col : (size_t)col;
+        wreg[i] = (k_in && col < N) ? *reinterpret_cast<const bf16x8_t*>(W + row * K + kb + lane * 8) : zero;
     };
-    fetch(0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) fetch_row(0, i);
 
     // the wave's columns of x as B operands: lane (n, g) holds x[n][kb + 32j + 8g ..], rows beyond M as zeros
     bf16x8_t bx[SW_STEPS];
@@ -76,9 +75,13 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
 
     for (int t = 0; t < n_tiles; ++t) {
         SW_WAVE_SYNC();                                         // the tile before has been read out of the wave's LDS
+        // row by row: as soon as a row has arrived and gone into LDS, the same row of the next tile is
+        // asked for, so that the loads on their way never run out at a tile's end
 #pragma unroll
-        for (int i = 0; i < 16; ++i) *reinterpret_cast<bf16x8_t*>(&stage[i * SW_STRIDE + lane * 8]) = wreg[i];
-        if (t + 1 < n_tiles) fetch(t + 1);
+        for (int i = 0; i < 16; ++i) {
+            *reinterpret_cast<bf16x8_t*>(&stage[i * SW_STRIDE + lane * 8]) = wreg[i];
+            if (t + 1 < n_tiles) fetch_row(t + 1, i);
+        }
         SW_WAVE_SYNC();                                         // the tile is complete in LDS
         float4_t c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -133,16 +136,14 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
     const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
     bf16x8_t wreg[16];
-    auto fetch = [&](int t, int p) {
+    auto fetch_row = [&](int t, int p, int i) {
         const int k = p * SW_SPAN + kb + lane * 8;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int col = b + G * (t * COLS + (GATED ? (i & 7) : i));
-            const size_t row = (GATED && i >= 8) ? (size_t)N + col : (size_t)col;
-            wreg[i] = (k < K && col < N) ? *reinterpret_cast<const bf16x8_t*>(W + row * K + k) : zero;
-        }
+        const int col = b + G * (t * COLS + (GATED ? (i & 7) : i));
+        const size_t row = (GATED && i >= 8) ? (size_t)N + col : (size_t)col;
+        wreg[i] = (k < K && col < N) ? *reinterpret_cast<const bf16x8_t*>(W + row * K + k) : zero;
     };
-    fetch(0, 0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) fetch_row(0, 0, i);
 
     for (int t = 0; t < n_tiles; ++t) {
         float4_t c = {0.f, 0.f, 0.f, 0.f};
@@ -154,10 +155,13 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
                 bx[j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
             }
             SW_WAVE_SYNC();
+            const bool more = p + 1 < spans || t + 1 < n_tiles;
+            const int t_next = p + 1 < spans ? t : t + 1, p_next = p + 1 < spans ? p + 1 : 0;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) *reinterpret_cast<bf16x8_t*>(&stage[i * SW_STRIDE + lane * 8]) = wreg[i];
-            if (p + 1 < spans) fetch(t, p + 1);
-            else if (t + 1 < n_tiles) fetch(t + 1, 0);
+            for (int i = 0; i < 16; ++i) {
+                *reinterpret_cast<bf16x8_t*>(&stage[i * SW_STRIDE + lane * 8]) = wreg[i];
+                if (more) fetch_row(t_next, p_next, i);
+            }
             SW_WAVE_SYNC();
 #pragma unroll
             for (int j = 0; j < SW_STEPS; ++j) {
