@@ -1,4 +1,4 @@
-// y = x @ W^T for up to 16 rows of x with W read as one sweep through memory: the decode-time
+// y = x @ W^T for up to 16 rows of x (32 with K up to 4,096) with W read as one sweep through memory: the decode-time
 // product of a small batch, which is bound by reading W once.
 // Layout as in the reference's F.linear (rollout/monkey_patch/qwen3.py:21): x [M, K], W [N, K],
 // y [M, N].
@@ -39,14 +39,17 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
         __builtin_amdgcn_wave_barrier();                         \
     } while (0)
 
-template <bool GATED, typename TO>
+// MB: blocks of 16 rows of x (1 or 2)
+template <int MB, bool GATED, typename TO>
 __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ W, TO* __restrict__ out, int M, int N, int K) {
     constexpr int COLS = GATED ? 8 : 16;                        // result columns of a tile
+    constexpr int RS = 16 * MB + 1;                             // row stride of the waves' tiles in LDS (floats)
+    constexpr bool TWO_BUFFERS = MB == 1;                       // of those tiles (LDS has room for one set with MB == 2)
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + (size_t)wave * 16 * SW_STRIDE;
-    float* red_both = reinterpret_cast<float*>(lds_raw + (size_t)SW_WAVES * 16 * SW_STRIDE * 2);   // [2][wave][16 rows][17]
+    float* red_both = reinterpret_cast<float*>(lds_raw + (size_t)SW_WAVES * 16 * SW_STRIDE * 2);   // [1 or 2][wave][16 rows][RS]
     const int G = gridDim.x, b = blockIdx.x;
     const int my_cols = N > b ? (N - 1 - b) / G + 1 : 0;
     const int n_tiles = (my_cols + COLS - 1) / COLS;
@@ -66,12 +69,14 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
     for (int i = 0; i < 16; ++i) fetch_row(0, i);
 
     // the wave's columns of x as B operands: lane (n, g) holds x[n][kb + 32j + 8g ..], rows beyond M as zeros
-    bf16x8_t bx[SW_STEPS];
+    bf16x8_t bx[MB][SW_STEPS];
 #pragma unroll
-    for (int j = 0; j < SW_STEPS; ++j) {
-        const int k = kb + 32 * j + 8 * g;
-        bx[j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
-    }
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int j = 0; j < SW_STEPS; ++j) {
+            const int k = kb + 32 * j + 8 * g, m = 16 * mb + n;
+            bx[mb][j] = (m < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)m * K + k) : zero;
+        }
 
     for (int t = 0; t < n_tiles; ++t) {
         SW_WAVE_SYNC();                                         // the tile before has been read out of the wave's LDS
@@ -83,36 +88,43 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
             if (t + 1 < n_tiles) fetch_row(t + 1, i);
         }
         SW_WAVE_SYNC();                                         // the tile is complete in LDS
-        float4_t c = {0.f, 0.f, 0.f, 0.f};
+        float4_t c[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) c[mb] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < SW_STEPS; ++j) {
             const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&stage[n * SW_STRIDE + 32 * j + 8 * g]);
-            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bx[j], c, 0, 0, 0);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) c[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bx[mb][j], c[mb], 0, 0, 0);
         }
         MFMA_SETTLE();
-        // c[i] = partial y[m = n][tile row 4g + i]: every wave puts its tile down, then the threads add
-        // the waves' tiles in wave order. Two buffers in turn: a buffer is written again two tiles on,
-        // which is after the next tile's barrier, and that its readers reach only when they have read.
-        float* red = red_both + (t & 1) * (SW_WAVES * 16 * 17);
+        // c[mb][i] = partial y[m = 16 mb + n][tile row 4g + i]: every wave puts its tile down, then the
+        // threads add the waves' tiles in wave order. With two buffers in turn a buffer is written again
+        // two tiles on, which is after the next tile's barrier, and that its readers reach only when
+        // they have read; with one, a second barrier ends the tile.
+        float* red = red_both + (TWO_BUFFERS ? (t & 1) * (SW_WAVES * 16 * RS) : 0);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) red[(wave * 16 + 4 * g + i) * 17 + n] = c[i];
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[(wave * 16 + 4 * g + i) * RS + 16 * mb + n] = c[mb][i];
         __syncthreads();
-        if (tid < 16 * COLS) {
+        if (tid < 16 * MB * COLS) {
             const int mm = tid / COLS, r = tid % COLS;        // r fastest: neighbours write neighbours' columns
             const int col = b + G * (t * COLS + r);
             if (mm < M && col < N) {
                 float s = 0.f;
 #pragma unroll
-                for (int w = 0; w < SW_WAVES; ++w) s += red[(w * 16 + r) * 17 + mm];
+                for (int w = 0; w < SW_WAVES; ++w) s += red[(w * 16 + r) * RS + mm];
                 if constexpr (GATED) {
                     float up = 0.f;
 #pragma unroll
-                    for (int w = 0; w < SW_WAVES; ++w) up += red[(w * 16 + 8 + r) * 17 + mm];
+                    for (int w = 0; w < SW_WAVES; ++w) up += red[(w * 16 + 8 + r) * RS + mm];
                     s = s / (1.0f + expf(-s)) * up;           // gate and up stay 32-bit until here
                 }
                 out[(size_t)mm * N + col] = from_f<TO>(s);
             }
         }
+        if constexpr (!TWO_BUFFERS) __syncthreads();
     }
 }
 
@@ -193,11 +205,14 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
     }
 }
 
+// the waves' W tiles, and their result tiles: two sets of 17 columns or one of 33
 static size_t sweep_lds() { return (size_t)SW_WAVES * 16 * SW_STRIDE * 2 + (size_t)2 * SW_WAVES * 16 * 17 * 4; }
 
-// Whether the sweep takes x [M, K]: up to 16 rows, K in whole pieces of 8 up to 8 spans.
+// Whether the sweep takes x [M, K]: up to 32 rows with K within one span, up to 16 rows with K up to
+// 8 spans, K in whole pieces of 8.
 extern "C" int ra_gemm_sweep_fits(int M, int K) {
-    return M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && K <= 8 * SW_SPAN;
+    if (M < 1 || K <= 0 || K % 8 != 0) return 0;
+    return K <= SW_SPAN ? M <= 32 : (M <= 16 && K <= 8 * SW_SPAN);
 }
 
 template <bool GATED, typename TO>
@@ -214,7 +229,19 @@ static int launch_sweep(int grid, hipStream_t st, const bf16* x, const bf16* W, 
         hipLaunchKernelGGL(long_kern, dim3(grid), dim3(SW_THREADS), sweep_lds(), st, x, W, out, M, N, K);
         return RA_OK;
     }
-    auto kern = gemm_sweep_kernel<GATED, TO>;
+    if (M > 16) {
+        auto wide_kern = gemm_sweep_kernel<2, GATED, TO>;
+        static bool wide_allowed = false;
+        if (!wide_allowed) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(wide_kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)sweep_lds()) != hipSuccess)
+                return RA_ERR_ARG;
+            wide_allowed = true;
+        }
+        hipLaunchKernelGGL(wide_kern, dim3(grid), dim3(SW_THREADS), sweep_lds(), st, x, W, out, M, N, K);
+        return RA_OK;
+    }
+    auto kern = gemm_sweep_kernel<1, GATED, TO>;
     static bool allowed = false;                              // per instantiation: more than 64 KB of LDS
     if (!allowed) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -145,6 +145,8 @@ class HipOps:
         a workgroup, K = 12,288) the library."""
         if not self.lib.ra_gemm_sweep_fits(M, K):
             return False
+        if M > 16 and not gated:             # 17 to 32 rows: 41 to 44 µs against the library's 49 and the SiLU-mul's 5
+            return False                     # for gate-up, but q/k/v 17 to 19 against 15, o 14 to 16 against 13
         rows = N * (2 if gated else 1)
         least = 8 if K <= 4096 else 32                   # rows a workgroup, at least
         return least * self.cu_count <= rows <= 256 * self.cu_count

@@ -229,12 +229,12 @@ def test_product_that_sweeps_the_weight(ops, N, K, gated):
     """The product that reads W as one sweep (column c with workgroup c % CUs): widths that fill
     every wave's 512 columns and widths that leave waves idle, widths of several spans of 4,096 (whole
     ones and one that ends after 8 columns), column counts that are no multiple of
-    the workgroups or of a tile, fewer columns than workgroups, 1 to 16 rows, both result types, the
+    the workgroups or of a tile, fewer columns than workgroups, 1 to 32 rows, both result types, the
     gated form; and what it does not take is refused."""
     from return_amd.kernels.hip_ops import _code, _ptr
     lib, st = ops.lib, torch.cuda.current_stream().cuda_stream
     w = rnd((2 if gated else 1) * N, K, dtype=torch.bfloat16, seed=N, scale=0.05)
-    for M in (1, 2, 5, 8, 13, 16):
+    for M in (1, 2, 5, 8, 13, 16) + ((17, 24, 32) if K <= 4096 else ()):
         x = rnd(M, K, dtype=torch.bfloat16, seed=M + 1)
         want = x.double() @ w.double().t()
         if gated:
@@ -248,11 +248,12 @@ def test_product_that_sweeps_the_weight(ops, N, K, gated):
                     torch.testing.assert_close(y.double(), want, atol=1e-4 * K ** 0.5, rtol=1e-5)
                 else:
                     torch.testing.assert_close(y.float(), want.float(), **tol(torch.bfloat16))
-    y = torch.empty(17, N, dtype=torch.bfloat16, device=DEV)
-    x = rnd(17, K, dtype=torch.bfloat16)
-    assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), 17, N, K, int(gated), _code(torch.bfloat16), 256, st) != 0
+    too_many = 33 if K <= 4096 else 17
+    y = torch.empty(too_many, N, dtype=torch.bfloat16, device=DEV)
+    x = rnd(too_many, K, dtype=torch.bfloat16)
+    assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), too_many, N, K, int(gated), _code(torch.bfloat16), 256, st) != 0
     assert lib.ra_gemm_sweep_fits(8, 4104) and not lib.ra_gemm_sweep_fits(8, 4100) and lib.ra_gemm_sweep_fits(16, 32768)
-    assert not lib.ra_gemm_sweep_fits(8, 32776)
+    assert not lib.ra_gemm_sweep_fits(8, 32776) and lib.ra_gemm_sweep_fits(32, 4096) and not lib.ra_gemm_sweep_fits(17, 4104)
     if gated:
         assert lib.ra_gemm_sweep_bf16(_ptr(x), _ptr(w), _ptr(y), 8, N, K, 1, _code(torch.float32), 256, st) != 0
 
