@@ -148,7 +148,7 @@ class HipOps:
         if M > 16 and not gated:             # 17 to 32 rows: 41 to 44 µs against the library's 49 and the SiLU-mul's 5
             return False                     # for gate-up, but q/k/v 17 to 19 against 15, o 14 to 16 against 13
         rows = N * (2 if gated else 1)
-        least = 8 if K <= 4096 else 32                   # rows a workgroup, at least
+        least = 8 if K <= 4096 or M <= 2 else 32         # rows a workgroup, at least (down at 1 and 2 rows: 20 against 21 to 23 µs)
         return least * self.cu_count <= rows <= 256 * self.cu_count
 
     def use_resident(self, M, N, K, gated):
