@@ -243,7 +243,7 @@ void attn_decode_kernel(
         const int kpos = max(min(max(c + lane, rg.lo), key_hi), start);
         const int idx = kpos - start;
         const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
-        return pt[pi] * P + (idx - pi * P);
+        return (pt[pi] * Hkv + kvh) * P + (idx - pi * P);     // [page][kv head][row in page]: this head's row
     };
     int row_next = 0;
     if constexpr (FUSED) {
@@ -265,7 +265,7 @@ void attn_decode_kernel(
             // head, each of their waves writes the same bits.
             const int idx = pos_q - start;
             const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
-            const size_t row_new = (size_t)pt[pi] * P + (idx - pi * P);
+            const size_t row_new = ((size_t)pt[pi] * Hkv + kvh) * P + (idx - pi * P);
             bf16x8_t kn[D32];
             const bf16* kp = tok + (size_t)(Hq + kvh) * D;
 #pragma unroll
@@ -276,12 +276,12 @@ void attn_decode_kernel(
             if (n == 0) {                                   // one lane of each g holds every piece once
 #pragma unroll
                 for (int j = 0; j < D32; ++j) {
-                    *reinterpret_cast<bf16x8_t*>(fz.k_out + (row_new * Hkv + kvh) * D + 32 * j + 8 * g) = kn[j];
+                    *reinterpret_cast<bf16x8_t*>(fz.k_out + row_new * D + 32 * j + 8 * g) = kn[j];
                     *reinterpret_cast<bf16x8_t*>(&new_s[32 * j + 8 * g]) = kn[j];
                 }
             }
             if (lane < LPR) {
-                *reinterpret_cast<uint4_t*>(fz.v_out + (row_new * Hkv + kvh) * D + lane * 8) = vn;
+                *reinterpret_cast<uint4_t*>(fz.v_out + row_new * D + lane * 8) = vn;
                 *reinterpret_cast<uint4_t*>(&new_s[D + lane * 8]) = vn;
             }
         }
@@ -314,7 +314,7 @@ void attn_decode_kernel(
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             const int r = __shfl(row, st * 16 + n, 64);
-            const bf16* kp = k_pool + ((size_t)r * Hkv + kvh) * D;
+            const bf16* kp = k_pool + (size_t)r * D;
 #pragma unroll
             for (int j = 0; j < D32; ++j)
                 ak[st][j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
@@ -329,7 +329,7 @@ void attn_decode_kernel(
         for (int i = 0; i < NVL; ++i) {
             const int e = min(lane + 64 * i, DEC_CHUNK * LPR - 1);
             const int r = __shfl(row, e / LPR, 64);
-            vv[i] = *reinterpret_cast<const uint4_t*>(v_pool + ((size_t)r * Hkv + kvh) * D + (e % LPR) * 8);
+            vv[i] = *reinterpret_cast<const uint4_t*>(v_pool + (size_t)r * D + (e % LPR) * 8);
         }
         WAVE_SYNC();                               // the previous pass has read its value tile
 #pragma unroll

@@ -130,12 +130,12 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
                 const int idx = p - start;
                 const int pi = idx >= 0 ? idx / P : 0;
                 const bool there = p >= lo_pos && p <= hi_pos && pi < n_listed;   // else: not a key of this pass
-                const int row = there ? pt[pi] * P + (idx - pi * P) : -1;
+                const int row = there ? (pt[pi] * Hkv + kvh) * P + (idx - pi * P) : -1;   // [page][kv head][row in page]
                 float dot[QR];
 #pragma unroll
                 for (int r = 0; r < QR; ++r) dot[r] = 0.f;
                 if (there) {
-                    const T* kr = k_pool + ((size_t)row * Hkv + kvh) * D;
+                    const T* kr = k_pool + (size_t)row * D;
                     if (vec) {
                         for (int j = part; 4 * j < D; j += 4) {
                             float kv[4];
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
 #pragma unroll 4
             for (int kk = 0; kk < nk; ++kk) {
                 const int row = max(my_row[kk], 0);      // a key that is not there has probability 0
-                const T* vr = v_pool + ((size_t)row * Hkv + kvh) * D;
+                const T* vr = v_pool + (size_t)row * D;
                 float pv[QR];
 #pragma unroll
                 for (int r = 0; r < QR; ++r) pv[r] = my_p[r * 64 + kk];

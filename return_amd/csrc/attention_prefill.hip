@@ -163,11 +163,11 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
     ([&]() {                                                                        \
         const int idx_ = min(max((kp), first_key), tile_last_pos) - start;          \
         const int pi_ = p_shift >= 0 ? (idx_ >> p_shift) : (idx_ / P);              \
-        return pt[pi_] * P + (idx_ - pi_ * P);                                      \
+        return (pt[pi_] * Hkv + kvh) * P + (idx_ - pi_ * P);                        \
     }())
 #define FETCH_ROW(row_)                                                             \
     {                                                                               \
-        const size_t base_ = ((size_t)(row_) * Hkv + kvh) * D;                      \
+        const size_t base_ = (size_t)(row_) * D;                                    \
         _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                           \
             const int p_ = my_sub + TPK * i;                                        \
             if (p_ < LPR) {                                                         \

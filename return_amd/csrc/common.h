@@ -89,6 +89,14 @@ __device__ __forceinline__ float rows_sum(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// The cache pools are [page][kv head][row in page][D]: the rows that one kv head has in a page lie
+// side by side, so that a kernel that walks through the keys of one kv head reads runs of P rows.
+// Offset (elements) of the row with slot number page * P + row in page, for kv head kvh.
+__host__ __device__ __forceinline__ size_t ra_cache_offset(long long slot, int kvh, int Hkv, int P, int D) {
+    const long long page = slot / P;
+    return (((size_t)page * Hkv + kvh) * P + (size_t)(slot - page * P)) * D;
+}
+
 static inline int ra_launch_status() {
     return hipGetLastError() == hipSuccess ? RA_OK : RA_ERR_LAUNCH;
 }

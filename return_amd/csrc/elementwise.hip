@@ -264,28 +264,32 @@ extern "C" int ra_split_heads(const void* qkv, void* q, void* k, void* v, int T_
 template <typename T>
 __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
                                 T* __restrict__ k_pool, T* __restrict__ v_pool,
-                                const int* __restrict__ slots, int W, long long pool_rows) {
+                                const int* __restrict__ slots, int Hkv, int D, int P, long long pool_rows) {
     const int t = blockIdx.x;
     const long long s = slots[t];
     if (s < 0 || s >= pool_rows) return;        // tables are built on the host; never write outside the pool
+    const int W = Hkv * D;
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        k_pool[s * W + c] = k[(size_t)t * W + c];
-        v_pool[s * W + c] = v[(size_t)t * W + c];
+        const int kvh = c / D;
+        const size_t at = ra_cache_offset(s, kvh, Hkv, P, D) + (c - kvh * D);
+        k_pool[at] = k[(size_t)t * W + c];
+        v_pool[at] = v[(size_t)t * W + c];
     }
 }
 
 extern "C" int ra_kv_write(const void* k, const void* v, void* k_pool, void* v_pool,
-                           const int* slots, int T_tokens, int W, long long pool_rows, int dtype,
+                           const int* slots, int T_tokens, int Hkv, int D, int P, long long pool_rows, int dtype,
                            void* stream) {
     if (T_tokens <= 0) return RA_OK;
+    if (Hkv <= 0 || D <= 0 || P <= 0) return RA_ERR_ARG;
     dim3 grid(T_tokens), block(256);
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, (hipStream_t)stream,
                            (const float*)k, (const float*)v, (float*)k_pool, (float*)v_pool, slots,
-                           W, pool_rows);
+                           Hkv, D, P, pool_rows);
     else
         hipLaunchKernelGGL(kv_write_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
-                           (const bf16*)k, (const bf16*)v, (bf16*)k_pool, (bf16*)v_pool, slots, W,
+                           (const bf16*)k, (const bf16*)v, (bf16*)k_pool, (bf16*)v_pool, slots, Hkv, D, P,
                            pool_rows);
     return ra_launch_status();
 }
@@ -302,7 +306,7 @@ __global__ void qkv_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, i
                                    float eps, const int* __restrict__ positions,
                                    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                    int R, T* __restrict__ q_out, T* __restrict__ k_pool,
-                                   T* __restrict__ v_pool, const int* __restrict__ slots,
+                                   T* __restrict__ v_pool, const int* __restrict__ slots, int P,
                                    long long pool_rows, long long n_rows) {
     const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= n_rows) return;
@@ -326,7 +330,7 @@ __global__ void qkv_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, i
         if (pool == nullptr) return;
         const long long s = slots[t];
         if (s < 0 || s >= pool_rows) return;
-        dst = pool + ((size_t)s * Hkv + kvh) * D;
+        dst = pool + ra_cache_offset(s, kvh, Hkv, P, D);
         if (is_k) {
             w = wk;
             rotate = R > 0;
@@ -397,7 +401,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_bf16x8_kernel(
     const bf16* __restrict__ qkv, int Hq, int Hkv, int D, const float* __restrict__ wq,
     const float* __restrict__ wk, float eps, const int* __restrict__ positions,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int R, bf16* __restrict__ q_out,
-    bf16* __restrict__ k_pool, bf16* __restrict__ v_pool, const int* __restrict__ slots,
+    bf16* __restrict__ k_pool, bf16* __restrict__ v_pool, const int* __restrict__ slots, int P,
     long long pool_rows, long long n_rows) {
     const long long row = ((long long)blockIdx.x * 256 + threadIdx.x) / GP;      // (token, head)
     const int sub = threadIdx.x % GP;
@@ -422,7 +426,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_bf16x8_kernel(
             const bool is_k = head < Hq + Hkv;
             bf16* pool = is_k ? k_pool : v_pool;
             const long long s = slots[t];
-            if (pool != nullptr && s >= 0 && s < pool_rows) dst = pool + ((size_t)s * Hkv + kvh) * D;
+            if (pool != nullptr && s >= 0 && s < pool_rows) dst = pool + ra_cache_offset(s, kvh, Hkv, P, D);
             if (is_k) {
                 w = wk;
                 rotate = R > 0;
@@ -491,18 +495,19 @@ template <int GP>
 static void launch_qkv_prepare_x8(long long n_rows, hipStream_t st, const bf16* qkv, int Hq, int Hkv, int D,
                                   const float* wq, const float* wk, float eps, const int* positions,
                                   const float* cos_t, const float* sin_t, int R, bf16* q_out, bf16* k_pool,
-                                  bf16* v_pool, const int* slots, long long pool_rows) {
+                                  bf16* v_pool, const int* slots, int P, long long pool_rows) {
     const long long threads = n_rows * GP;
     hipLaunchKernelGGL(qkv_prepare_bf16x8_kernel<GP>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
                        st, qkv, Hq, Hkv, D, wq, wk, eps, positions, cos_t, sin_t, R, q_out, k_pool, v_pool,
-                       slots, pool_rows, n_rows);
+                       slots, P, pool_rows, n_rows);
 }
 
 extern "C" int ra_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, int D, const float* wq,
                               const float* wk, float eps, const int* positions, const float* cos_t,
                               const float* sin_t, int R, void* q_out, void* k_pool, void* v_pool,
-                              const int* slots, long long pool_rows, int dtype, void* stream) {
+                              const int* slots, int P, long long pool_rows, int dtype, void* stream) {
     if (T_tokens <= 0) return RA_OK;
+    if ((k_pool != nullptr || v_pool != nullptr) && P <= 0) return RA_ERR_ARG;
     if (D > 64 * QKV_MAX_PER_LANE * 2 || R > D || (R & 1)) return RA_ERR_ARG;
     // pairs: R/2 <= 256; pass-through: D-R <= 256
     if ((R >> 1) > 64 * QKV_MAX_PER_LANE || (D - R) > 64 * QKV_MAX_PER_LANE) return RA_ERR_ARG;
@@ -512,7 +517,7 @@ extern "C" int ra_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, in
 #define QKV_X8(GP)                                                                                    \
     launch_qkv_prepare_x8<GP>(n_rows, (hipStream_t)stream, (const bf16*)qkv, Hq, Hkv, D, wq, wk, eps,  \
                               positions, cos_t, sin_t, R, (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool,  \
-                              slots, pool_rows)
+                              slots, P, pool_rows)
         if (lanes <= 1) QKV_X8(1);
         else if (lanes <= 2) QKV_X8(2);
         else if (lanes <= 4) QKV_X8(4);
@@ -526,11 +531,11 @@ extern "C" int ra_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, in
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(qkv_prepare_kernel<float>, grid, block, 0, (hipStream_t)stream,
                            (const float*)qkv, Hq, Hkv, D, wq, wk, eps, positions, cos_t, sin_t, R,
-                           (float*)q_out, (float*)k_pool, (float*)v_pool, slots, pool_rows, n_rows);
+                           (float*)q_out, (float*)k_pool, (float*)v_pool, slots, P, pool_rows, n_rows);
     else
         hipLaunchKernelGGL(qkv_prepare_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
                            (const bf16*)qkv, Hq, Hkv, D, wq, wk, eps, positions, cos_t, sin_t, R,
-                           (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, pool_rows, n_rows);
+                           (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, P, pool_rows, n_rows);
     return ra_launch_status();
 }
 

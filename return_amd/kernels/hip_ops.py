@@ -55,8 +55,8 @@ def _declare(lib):
         "ra_head_rmsnorm": [P, P, F, L, I, I, P],
         "ra_rope": [P, P, P, P, I, I, I, I, I, P],
         "ra_split_heads": [P, P, P, P, I, I, I, I, P],
-        "ra_kv_write": [P, P, P, P, P, I, I, L, I, P],
-        "ra_qkv_prepare": [P, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, L, I, P],
+        "ra_kv_write": [P, P, P, P, P, I, I, I, I, L, I, P],
+        "ra_qkv_prepare": [P, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, I, L, I, P],
         "ra_silu_mul": [P, P, I, I, I, P],
         "ra_gemm_nt": [P, P, P, I, I, I, I, I, P],
         "ra_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, P],
@@ -255,13 +255,17 @@ class HipOps:
                                             _code(qkv.dtype), self._stream()), "split_heads")
 
     def _pool_rows(self, k_pool, v_pool, n_kv, D, dtype):
+        """Checks the pools of one cache layer, [pages, kv heads, rows in a page, D], and returns the
+        number of token rows they hold (pages x page size)."""
         for t, name in ((k_pool, "k pool"), (v_pool, "v pool")):
             self._want(t, name, dtype, 4)
-            if t.shape[2] != n_kv or t.shape[3] != D:
+            if t.shape[1] != n_kv or t.shape[3] != D:
                 raise KernelError(f"{name} {tuple(t.shape)} does not hold {n_kv} heads of {D}")
         if k_pool.shape != v_pool.shape:
             raise KernelError("k pool and v pool differ in shape")
-        return k_pool.shape[0] * k_pool.shape[1]
+        if k_pool.shape[0] * k_pool.shape[1] * k_pool.shape[2] >= 2 ** 31:
+            raise KernelError(f"k pool {tuple(k_pool.shape)}: the kernels count head rows in 32 bits")
+        return k_pool.shape[0] * k_pool.shape[2]
 
     def kv_write(self, k, v, k_pool, v_pool, slot_mapping):
         self._want(k, "k", dims=3)
@@ -272,7 +276,7 @@ class HipOps:
         if v.shape != k.shape or slot_mapping.shape[0] != T:
             raise KernelError(f"kv_write: k {tuple(k.shape)}, v {tuple(v.shape)}, slots {tuple(slot_mapping.shape)}")
         self._check(self.lib.ra_kv_write(_ptr(k), _ptr(v), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping),
-                                         T, n_kv * D, rows, _code(k.dtype), self._stream()), "kv_write")
+                                         T, n_kv, D, k_pool.shape[2], rows, _code(k.dtype), self._stream()), "kv_write")
 
     def qkv_prepare(self, qkv, n_q, n_kv, D, w_q, w_k, eps, positions, cos, sin, rotary_dim, q_out,
                     k_pool, v_pool, slot_mapping):
@@ -306,7 +310,8 @@ class HipOps:
         self._check(self.lib.ra_qkv_prepare(
             _ptr(qkv), T, n_q, n_kv, D, _ptr(w_q), _ptr(w_k), float(eps), _ptr(positions),
             _ptr(cos) if R else None, _ptr(sin) if R else None, R, _ptr(q_out), _ptr(k_pool),
-            _ptr(v_pool), _ptr(slot_mapping), rows, _code(qkv.dtype), self._stream()), "qkv_prepare")
+            _ptr(v_pool), _ptr(slot_mapping), k_pool.shape[2] if k_pool is not None else 0, rows, _code(qkv.dtype),
+            self._stream()), "qkv_prepare")
 
     def silu_mul(self, gu, out):
         self._want(gu, "gate-up", dims=2)
@@ -517,7 +522,7 @@ class HipOps:
         self._want(out, "attention output", q.dtype, 3)
         T, n_q, D = q.shape
         g = step.groups[group]
-        n_kv = k_pool.shape[2]
+        n_kv = k_pool.shape[1]
         self._pool_rows(k_pool, v_pool, n_kv, D, q.dtype)
         if out.shape != q.shape or T != step.n_tokens:
             raise KernelError(f"attention: q {tuple(q.shape)}, out {tuple(out.shape)}, step of {step.n_tokens}")
@@ -525,7 +530,7 @@ class HipOps:
             raise KernelError(f"attention: {n_q} query heads over {n_kv} kv heads")
         if D > 512:
             raise KernelError(f"attention: head size {D} is beyond the kernel's 512")
-        P = k_pool.shape[1]
+        P = k_pool.shape[2]
         window = int(window)
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
         fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
@@ -620,7 +625,7 @@ class HipOps:
             self._want(sin, "sin table", torch.float32, 2)
             if cos.shape[1] != D // 2 or sin.shape != cos.shape:
                 raise KernelError(f"attention_qkv: tables {tuple(cos.shape)} for head size {D}")
-        P = k_pool.shape[1]
+        P = k_pool.shape[2]
         window = int(window)
         S, max_splits, merge = self._decode_splits(step, n_q, n_kv, D, window)
         nd = step.n_decode

@@ -190,8 +190,8 @@ def test_groups_have_pools_of_their_own():
     assert sorted(map(tuple, (g.layers for g in cm.groups))) == [(0, 3), (1,), (2,)]
     v0, v3 = cm.view(0), cm.view(3)
     assert v0.group == v3.group and v0.k_pool.data_ptr() != v3.k_pool.data_ptr()
-    # 32 tokens in pages of 4, and the spare page
-    assert v0.k_pool.shape == (8 + 1, 4, 2, 8) and cm.view(2).k_pool.shape == (8 + 1, 4, 1, 16)
+    # 32 tokens in pages of 4, and the spare page; [pages, kv heads, rows in a page, D]
+    assert v0.k_pool.shape == (8 + 1, 2, 4, 8) and cm.view(2).k_pool.shape == (8 + 1, 1, 4, 16)
 
 
 def test_pad_tables_adds_rows_on_the_spare_page_only():

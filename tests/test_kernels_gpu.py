@@ -117,7 +117,7 @@ def test_qkv_prepare(ops, ref, dtype, Hq, Hkv, D, R, norm):
     outs = []
     for o in (ops, ref):
         q = torch.zeros(T, Hq, D, dtype=dtype, device=DEV)
-        kp = torch.zeros(pages, P, Hkv, D, dtype=dtype, device=DEV)
+        kp = torch.zeros(pages, Hkv, P, D, dtype=dtype, device=DEV)
         vp = torch.zeros_like(kp)
         o.qkv_prepare(qkv, Hq, Hkv, D, wq, wk, 1e-6, pos, cos, sin, R, q, kp, vp, slots)
         outs.append((q, kp, vp))
@@ -140,7 +140,7 @@ def test_split_and_kv_write(ops, ref, dtype):
         k = torch.empty(T, Hkv, D, dtype=dtype, device=DEV)
         v = torch.empty_like(k)
         o.split_heads(qkv, Hq, Hkv, D, q, k, v)
-        kp = torch.zeros(pages, P, Hkv, D, dtype=dtype, device=DEV)
+        kp = torch.zeros(pages, Hkv, P, D, dtype=dtype, device=DEV)
         vp = torch.zeros_like(kp)
         o.kv_write(k, v, kp, vp, slots)
         res.append((q, k, v, kp, vp))
@@ -446,8 +446,8 @@ def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
     for k in need:
         pages_of.append([perm.pop() for _ in range(k)])
     step = _step(q_lens, q_starts, P, pages_of)
-    kp = rnd(total_pages, P, Hkv, D, dtype=dtype, seed=51)
-    vp = rnd(total_pages, P, Hkv, D, dtype=dtype, seed=52)
+    kp = rnd(total_pages, Hkv, P, D, dtype=dtype, seed=51)
+    vp = rnd(total_pages, Hkv, P, D, dtype=dtype, seed=52)
     q = rnd(sum(q_lens), Hq, D, dtype=dtype, seed=53)
     a = torch.zeros_like(q)
     b = torch.zeros_like(q)
@@ -472,8 +472,8 @@ def test_prefill_attention_every_head_size(ops, ref, D, key_split, monkeypatch):
             pages_of.append(list(range(nxt, nxt + k)))
             nxt += k
         step = _step([s[0] for s in segs], [s[1] for s in segs], P, pages_of)
-        kp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D)
-        vp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D + 1)
+        kp = rnd(nxt, Hkv, P, D, dtype=torch.bfloat16, seed=D)
+        vp = rnd(nxt, Hkv, P, D, dtype=torch.bfloat16, seed=D + 1)
         q = rnd(sum(s[0] for s in segs), Hq, D, dtype=torch.bfloat16, seed=D + 2)
         a, b = torch.zeros_like(q), torch.zeros_like(q)
         ops.attention(q, a, kp, vp, step, 0, D ** -0.5, window)
@@ -497,8 +497,8 @@ def test_decode_attention_every_head_size(ops, ref, monkeypatch, D, merge):
             pages_of.append(list(range(nxt, nxt + k)))
             nxt += k
         step = _step([1] * len(segs), [s[1] for s in segs], P, pages_of)
-        kp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D)
-        vp = rnd(nxt, P, Hkv, D, dtype=torch.bfloat16, seed=D + 1)
+        kp = rnd(nxt, Hkv, P, D, dtype=torch.bfloat16, seed=D)
+        vp = rnd(nxt, Hkv, P, D, dtype=torch.bfloat16, seed=D + 1)
         q = rnd(len(segs), Hq, D, dtype=torch.bfloat16, seed=D + 2)
         a, b = torch.zeros_like(q), torch.zeros_like(q)
         ops.attention(q, a, kp, vp, step, 0, D ** -0.5, 0)
@@ -528,11 +528,11 @@ def test_attention_edges_of_window_and_causality(ops, dtype, q_len, older_wins):
     k = torch.zeros(L, Hkv, D)
     k[:, :, 0] = mag[:, None]
     v = rnd(L, Hkv, D, seed=71).cpu()
-    kp = torch.zeros(n_pages + 5, P, Hkv, D)
+    kp = torch.zeros(n_pages + 5, Hkv, P, D)
     vp = torch.zeros_like(kp)
     for i in range(L):
-        kp[pages[i // P], i % P] = k[i]
-        vp[pages[i // P], i % P] = v[i]
+        kp[pages[i // P], :, i % P] = k[i]               # pools are [pages, kv heads, rows in a page, D]
+        vp[pages[i // P], :, i % P] = v[i]
     kp, vp = kp.to(dtype).to(DEV), vp.to(dtype).to(DEV)
     q = torch.zeros(q_len, Hq, D)
     q[:, :, 0] = 96.0                                    # 96 * 1 / sqrt(64) = 12 per step of the magnitude
@@ -553,14 +553,14 @@ def test_attention_far_key_stands_out(ops, dtype):
     Hq, Hkv, D, P, L = 4, 2, 64, 16, 700
     pages = list(range(-(-L // P)))
     step = _step([1], [L - 1], P, [pages])
-    kp = rnd(len(pages), P, Hkv, D, dtype=dtype, seed=61, scale=0.1)
-    vp = rnd(len(pages), P, Hkv, D, dtype=dtype, seed=62)
+    kp = rnd(len(pages), Hkv, P, D, dtype=dtype, seed=61, scale=0.1)
+    vp = rnd(len(pages), Hkv, P, D, dtype=dtype, seed=62)
     q = rnd(1, Hq, D, dtype=dtype, seed=63, scale=0.1)
     far = 37
-    kp.view(-1, Hkv, D)[far] = (q.view(Hq, D)[::2] * 400).to(dtype)      # kv head h gets query head 2h, scaled up
+    kp[far // P, :, far % P] = (q.view(Hq, D)[::2] * 400).to(dtype)      # kv head h gets query head 2h, scaled up
     out = torch.zeros_like(q)
     ops.attention(q, out, kp, vp, step, 0, 1.0, 0)
-    want = vp.view(-1, Hkv, D)[far].float()
+    want = vp[far // P, :, far % P].float()
     torch.testing.assert_close(out[0, ::2].float(), want, atol=3e-2, rtol=3e-2)
 
 
@@ -581,8 +581,8 @@ def test_decode_attention_that_prepares_q_k_v_itself(ops, monkeypatch, D, Hq, Hk
     pages_of = [[perm.pop() for _ in range(k)] for k in need]
     step = _step([1] * len(starts), starts, P, pages_of)
     n = len(starts)
-    kp = rnd(sum(need) + 3, P, Hkv, D, dtype=torch.bfloat16, seed=1)
-    vp = rnd(sum(need) + 3, P, Hkv, D, dtype=torch.bfloat16, seed=2)
+    kp = rnd(sum(need) + 3, Hkv, P, D, dtype=torch.bfloat16, seed=1)
+    vp = rnd(sum(need) + 3, Hkv, P, D, dtype=torch.bfloat16, seed=2)
     qkv = rnd(n, (Hq + 2 * Hkv) * D, dtype=torch.bfloat16, seed=3)
     wq = (1 + 0.1 * rnd(D, seed=4)) if normed else None
     wk = (1 + 0.1 * rnd(D, seed=5)) if normed else None
@@ -620,8 +620,8 @@ def test_attention_over_a_long_context(ops, ref, dtype):
     perm = torch.randperm(sum(need) + 7, generator=torch.Generator().manual_seed(3)).tolist()
     pages_of = [[perm.pop() for _ in range(k)] for k in need]
     step = _step([s[0] for s in segs], [s[1] for s in segs], P, pages_of)
-    kp = rnd(sum(need) + 7, P, Hkv, D, dtype=dtype, seed=81)
-    vp = rnd(sum(need) + 7, P, Hkv, D, dtype=dtype, seed=82)
+    kp = rnd(sum(need) + 7, Hkv, P, D, dtype=dtype, seed=81)
+    vp = rnd(sum(need) + 7, Hkv, P, D, dtype=dtype, seed=82)
     q = rnd(sum(s[0] for s in segs), Hq, D, dtype=dtype, seed=83)
     a, b = torch.zeros_like(q), torch.zeros_like(q)
     ops.attention(q, a, kp, vp, step, 0, D ** -0.5, 0)
@@ -702,14 +702,14 @@ def test_calls_that_do_not_fit_are_refused_before_anything_runs(ops):
     step = _step([1], [5], 16, [[0]])
     for Hq, Hkv, D, why in ((3, 2, 16, "heads"), (2, 2, 528, "head size")):
         q = rnd(1, Hq, D, dtype=bf)
-        kp = rnd(1, 16, Hkv, D, dtype=bf)
+        kp = rnd(1, Hkv, 16, D, dtype=bf)
         bad.append((f"attention: {why}", lambda q=q, kp=kp: ops.attention(q, torch.zeros_like(q), kp, kp.clone(), step, 0, 1.0, 0)))
     q = rnd(1, 4, 32, dtype=bf)
     bad.append(("attention: pool of another head size",
-                lambda: ops.attention(q, torch.zeros_like(q), rnd(1, 16, 2, 16, dtype=bf), rnd(1, 16, 2, 16, dtype=bf), step, 0, 1.0, 0)))
+                lambda: ops.attention(q, torch.zeros_like(q), rnd(1, 2, 16, 16, dtype=bf), rnd(1, 2, 16, 16, dtype=bf), step, 0, 1.0, 0)))
     bad.append(("attention: output of another shape",
-                lambda: ops.attention(q, torch.zeros(2, 4, 32, dtype=bf, device=DEV), rnd(1, 16, 2, 32, dtype=bf),
-                                      rnd(1, 16, 2, 32, dtype=bf), step, 0, 1.0, 0)))
+                lambda: ops.attention(q, torch.zeros(2, 4, 32, dtype=bf, device=DEV), rnd(1, 2, 16, 32, dtype=bf),
+                                      rnd(1, 2, 16, 32, dtype=bf), step, 0, 1.0, 0)))
     for name, call in bad:
         with pytest.raises(KernelError):
             call()

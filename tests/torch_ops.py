@@ -59,10 +59,10 @@ class TorchOps:
 
     # rollout/cache.py:334-337
     def kv_write(self, k, v, k_pool, v_pool, slot_mapping):
-        kf = k_pool.view(-1, k_pool.shape[2], k_pool.shape[3])
-        vf = v_pool.view(-1, v_pool.shape[2], v_pool.shape[3])
-        kf[slot_mapping.long()] = k
-        vf[slot_mapping.long()] = v
+        P = k_pool.shape[2]                                 # pools are [pages, kv heads, rows in a page, D]
+        page, row = slot_mapping.long() // P, slot_mapping.long() % P
+        k_pool[page, :, row] = k
+        v_pool[page, :, row] = v
 
     def qkv_prepare(self, qkv, n_q, n_kv, D, w_q, w_k, eps, positions, cos, sin, rotary_dim, q_out,
                     k_pool, v_pool, slot_mapping):
@@ -110,8 +110,7 @@ class TorchOps:
     # gathered as opd/test_parallel.py:14-42 does
     def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
         g = step.groups[group]
-        P = k_pool.shape[1]
-        n_q, n_kv = q.shape[1], k_pool.shape[2]
+        n_q, n_kv = q.shape[1], k_pool.shape[1]
         cu_q, cu_p = step.cu_q.tolist(), g.cu_pages.tolist()
         q_start, kv_start = step.q_start.tolist(), g.kv_start.tolist()
         table = g.page_table.long()
@@ -119,8 +118,8 @@ class TorchOps:
             a, b = cu_q[s], cu_q[s + 1]
             pages = table[cu_p[s]:cu_p[s + 1]]
             end = q_start[s] + (b - a)                      # keys held after this step
-            k = k_pool[pages].reshape(-1, n_kv, k_pool.shape[3])[:end - kv_start[s]].float()
-            v = v_pool[pages].reshape(-1, n_kv, v_pool.shape[3])[:end - kv_start[s]].float()
+            k = k_pool[pages].transpose(1, 2).reshape(-1, n_kv, k_pool.shape[3])[:end - kv_start[s]].float()
+            v = v_pool[pages].transpose(1, 2).reshape(-1, n_kv, v_pool.shape[3])[:end - kv_start[s]].float()
             k_pos = torch.arange(kv_start[s], end, device=q.device)
             q_pos = torch.arange(q_start[s], end, device=q.device)
             kk = k.repeat_interleave(n_q // n_kv, dim=1)
