@@ -260,7 +260,7 @@ extern "C" int ra_split_heads(const void* qkv, void* q, void* k, void* v, int T_
 }
 
 // ------------------------------------------------------------------ cache write
-// k, v: [T, Hkv*D] rows; pools: [rows, Hkv*D]; slot[t] = page*P + offset.
+// k, v: [T, Hkv*D] rows; pools: [pages, Hkv, P, D]; slot[t] = page*P + row in the page.
 template <typename T>
 __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
                                 T* __restrict__ k_pool, T* __restrict__ v_pool,
