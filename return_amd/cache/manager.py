@@ -67,6 +67,9 @@ class PagedGroup:
         # a page of one layer is one contiguous run of Hkv*P*D elements. One page beyond the
         # num_pages that requests can hold is the spare page: rows that only fill a batch up
         # to a fixed size (pad_tables) write and read there.
+        if (num_pages + 1) * page_size * spec.num_kv_heads >= 2 ** 31:
+            raise ValueError(f"{num_pages} pages of {page_size} rows for {spec.num_kv_heads} kv heads: the kernels "
+                             "count a layer's head rows in 32 bits")
         self.pool = torch.zeros(len(self.layers), 2, num_pages + 1, spec.num_kv_heads, page_size,
                                 spec.head_dim, dtype=dtype, device=device)
         self.spare_page = num_pages

@@ -233,3 +233,9 @@ def test_pool_bytes_is_what_the_manager_allocates():
         held = sum(g.pool.numel() * g.pool.element_size() for g in cm.groups)
         held += sum(t.numel() * t.element_size() for ts in cm.state.values() for t in ts.values())
         assert CacheManager.pool_bytes(layers, 4, 50, 3, dtype) == held
+
+
+def test_a_pool_whose_head_rows_do_not_fit_32_bits_is_refused():
+    with pytest.raises(ValueError, match="32 bits"):
+        CacheManager({0: PagedKVSpec(8, 128)}, page_size=16, max_token=2 ** 28, max_requests=1, dtype=torch.bfloat16,
+                     device="meta")
