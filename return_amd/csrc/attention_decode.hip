@@ -27,6 +27,10 @@
 // BUILD-VARIANTS: DEC_PART=0 DEC_PART=1 DEC_PART=2 DEC_PART=3 DEC_API=1
 // (each DEC_PART instantiates four head sizes; DEC_API holds the entry point and the merge)
 #include "common.h"
+#ifdef DEC_API
+#include <mutex>
+#include "no_alloc.h"
+#endif
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -667,5 +671,55 @@ extern "C" int ra_attention_decode_fused_bf16(const void* qkv, void* out, void* 
     return decode_launch(nullptr, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
                          Hkv, D, P, scale, window, split_tokens, max_splits, fz, merge, (hipStream_t)stream);
+}
+
+// ---- the entry point that allocates nothing (declared in no_alloc.h) ----
+// The partial sums live in a file-scope device array. In host code that name is a stand-in of the
+// host side, not a device address: the address on each GPU (every GPU has its own copy) is asked
+// for once per device with hipGetSymbolAddress and kept; only that pointer goes to kernels.
+static __device__ __align__(256) float ra_decode_scratch[RA_DECODE_STATIC_FLOATS];
+
+#define RA_MAX_DEVICES 64
+static std::mutex ra_scratch_lock;
+static float* ra_scratch_on_device[RA_MAX_DEVICES] = {};
+
+// The device array's address on the current device, or nullptr. Asked for at the first call on a device.
+static float* decode_scratch_here() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= RA_MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> hold(ra_scratch_lock);
+    if (ra_scratch_on_device[dev] == nullptr) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(ra_decode_scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        ra_scratch_on_device[dev] = (float*)p;
+    }
+    return ra_scratch_on_device[dev];
+}
+
+extern "C" int ra_attention_decode_static_bf16(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                               const int* page_table, const int* cu_pages,
+                                               const int* kv_start, const int* cu_q, const int* q_start,
+                                               const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
+                                               float scale, int window, int split_tokens, int max_splits,
+                                               int merge, void* stream) {
+    if (n_dec < 0 || Hq <= 0 || D <= 0 || max_splits <= 0) return RA_ERR_ARG;
+    float* pa = nullptr;
+    float* pm = nullptr;
+    if (!merge && n_dec > 0) {
+        const unsigned long long acc = (unsigned long long)n_dec * Hq * max_splits * D;
+        const unsigned long long ml = (unsigned long long)n_dec * Hq * max_splits * 2;
+        if (acc + ml > (unsigned long long)RA_DECODE_STATIC_FLOATS) return RA_ERR_SCRATCH;
+        float* base = decode_scratch_here();
+        if (base == nullptr) return RA_ERR_SETUP;
+        pa = base;                 // [n_dec, Hq, max_splits, D]
+        pm = base + acc;           // [n_dec, Hq, max_splits, 2]
+    }
+    DecodeFused none = {};
+    return decode_launch((const bf16*)q, out, pa, pm, (const bf16*)k_pool, (const bf16*)v_pool, page_table,
+                         cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq, Hkv, D, P, scale, window,
+                         split_tokens, max_splits, none, merge, (hipStream_t)stream);
 }
 #endif  // DEC_API

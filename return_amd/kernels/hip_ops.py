@@ -69,6 +69,7 @@ def _declare(lib):
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, I, P],
+        "ra_attention_decode_static_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_merge_waves": [I],
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "ra_attention_prefill_tile_rows": [I],
@@ -168,7 +169,9 @@ class HipOps:
 
     def _check(self, status: int, name: str):
         if status != 0:
-            why = {1: "arguments outside what the kernel takes", 2: "launch failed"}.get(status, "?")
+            why = {1: "arguments outside what the kernel takes", 2: "launch failed",
+                   3: "more partial results than the library's own buffer holds",
+                   4: "the library's own buffer was not found on this device"}.get(status, "?")
             raise KernelError(f"{name}: {why} (status {status})")
 
     def _want(self, t, name, dtype=None, dims=None):
