@@ -49,6 +49,10 @@ class StepTables:
     seq_lens: np.ndarray        # [n]   tokens held after this step
     slot_ids: np.ndarray        # [n]   the request's state slot
     groups: List[GroupTables]
+    # (version of the page lists, request ids[, rows that fill the batch up]): two steps with the same
+    # key have the same page_table, cu_pages and kv_start in every group, so whoever copies them to
+    # the device may skip that (rollout/cache.py:286-306 skips its table rebuild on the same test)
+    page_key: Optional[tuple] = None
 
 
 class PagedGroup:
@@ -151,6 +155,11 @@ class CacheManager:
         self.live: Dict[object, _Live] = {}
         self._step_requests: List = []
         self.version = 0            # changes whenever any request's page list changes
+        self._memo_key = None       # page_key of the last step and its groups' (page_table, cu_pages, kv_start)
+        self._memo_tables: List = []
+        self._pad_key = None        # the same for the last step that was filled up
+        self._pad_tables: List = []
+        self.table_builds = 0       # steps whose page tables were put together anew
 
     @staticmethod
     def pool_bytes(cache_layers: Dict[int, object], page_size: int, max_token: int, max_requests: int,
@@ -280,37 +289,48 @@ class CacheManager:
                 positions[cu_q[i]:cu_q[i + 1]] = np.arange(q_start[i], q_start[i] + q_lens[i])
         slot_ids = np.array([r.slot for r in lives], dtype=np.int32)
 
-        groups = []
         for g, grp in enumerate(self.groups):
-            slot_mapping = np.empty(total, dtype=np.int32)
-            cu_pages = np.zeros(n + 1, dtype=np.int32)
-            kv_start = np.zeros(n, dtype=np.int32)
-            tables = []
             for i, r in enumerate(lives):
                 need = self._need(r, g, q_lens[i])
                 if need:
                     r.pages[g].extend(grp.pages.take_many(need))
                     r.pages_changed(g)
                     self.version += 1
-                pages = r.pages_array(g)
+        # the page lists are final now: the same (version, requests) as the last step means the same tables
+        ids = [rid for rid, _ in entries]
+        page_key = (self.version, tuple(ids))
+        same = page_key == self._memo_key
+        if not same:
+            self.table_builds += 1
+            self._memo_tables = []
+
+        groups = []
+        for g, grp in enumerate(self.groups):
+            slot_mapping = np.empty(total, dtype=np.int32)
+            for i, r in enumerate(lives):
                 if single:
                     rel = r.seq_len - r.first_pos[g]
                     slot_mapping[i] = r.pages[g][rel // P] * P + rel % P
                 else:
                     rel = positions[cu_q[i]:cu_q[i + 1]] - r.first_pos[g]
-                    slot_mapping[cu_q[i]:cu_q[i + 1]] = pages[rel // P] * P + rel % P
-                tables.append(pages)
-                cu_pages[i + 1] = cu_pages[i] + len(pages)
-                kv_start[i] = r.first_pos[g]
-            page_table = np.concatenate(tables) if tables else np.zeros(0, dtype=np.int32)
+                    slot_mapping[cu_q[i]:cu_q[i + 1]] = r.pages_array(g)[rel // P] * P + rel % P
+            if same:
+                page_table, cu_pages, kv_start = self._memo_tables[g]
+            else:
+                tables = [r.pages_array(g) for r in lives]
+                cu_pages = np.zeros(n + 1, dtype=np.int32)
+                cu_pages[1:] = np.cumsum([len(t) for t in tables])
+                kv_start = np.array([r.first_pos[g] for r in lives], dtype=np.int32)
+                page_table = np.concatenate(tables) if tables else np.zeros(0, dtype=np.int32)
+                self._memo_tables.append((page_table, cu_pages, kv_start))
             groups.append(GroupTables(slot_mapping, page_table, cu_pages, kv_start))
+        self._memo_key = page_key
 
         for rid, n_new in entries:
             self.live[rid].seq_len += n_new
         seq_lens = np.array([self.live[rid].seq_len for rid, _ in entries], dtype=np.int32)
         self._step_requests = [rid for rid, _ in entries]
-        return StepTables([rid for rid, _ in entries], q_lens, q_start, cu_q, positions,
-                          seq_lens, slot_ids, groups)
+        return StepTables(ids, q_lens, q_start, cu_q, positions, seq_lens, slot_ids, groups, page_key)
 
     def pad_tables(self, tables: StepTables, n_pad: int) -> StepTables:
         """The same step with n_pad more one-token sequences that belong to no request: token
@@ -322,20 +342,30 @@ class CacheManager:
         P = self.page_size
         one = np.ones(n_pad, dtype=np.int32)
         last = int(tables.cu_q[-1])
+        page_key = None if tables.page_key is None else tables.page_key + (n_pad,)
+        same = page_key is not None and page_key == self._pad_key
+        if not same:
+            self._pad_tables = []
         groups = []
-        for grp, gt in zip(self.groups, tables.groups):
+        for g, (grp, gt) in enumerate(zip(self.groups, tables.groups)):
+            if same:
+                page_table, cu_pages, kv_start = self._pad_tables[g]
+            else:
+                page_table = np.concatenate([gt.page_table, one * grp.spare_page]).astype(np.int32)
+                cu_pages = np.concatenate([gt.cu_pages, gt.cu_pages[-1] + np.arange(1, n_pad + 1)]).astype(np.int32)
+                kv_start = np.concatenate([gt.kv_start, 0 * one]).astype(np.int32)
+                self._pad_tables.append((page_table, cu_pages, kv_start))
             groups.append(GroupTables(
                 np.concatenate([gt.slot_mapping, one * (grp.spare_page * P)]).astype(np.int32),
-                np.concatenate([gt.page_table, one * grp.spare_page]).astype(np.int32),
-                np.concatenate([gt.cu_pages, gt.cu_pages[-1] + np.arange(1, n_pad + 1)]).astype(np.int32),
-                np.concatenate([gt.kv_start, 0 * one]).astype(np.int32)))
+                page_table, cu_pages, kv_start))
+        self._pad_key = page_key
         return StepTables(
             list(tables.request_ids) + [None] * n_pad, list(tables.q_lens) + [1] * n_pad,
             np.concatenate([tables.q_start, 0 * one]).astype(np.int32),
             np.concatenate([tables.cu_q, last + np.arange(1, n_pad + 1)]).astype(np.int32),
             np.concatenate([tables.positions, 0 * one]).astype(np.int32),
             np.concatenate([tables.seq_lens, one]).astype(np.int32),
-            np.concatenate([tables.slot_ids, one * self.spare_slot]).astype(np.int32), groups)
+            np.concatenate([tables.slot_ids, one * self.spare_slot]).astype(np.int32), groups, page_key)
 
     def end_step(self) -> None:
         """After the step ran: give back pages that every later query's window has passed."""

@@ -5,7 +5,8 @@ The reference fills pinned host arrays and copies them into persistent device
 tensors so that captured graphs replay on fixed addresses (rollout/cache.py:42-70,
 274-328). Here all integer tables of a step live in ONE pinned staging buffer and
 ONE device buffer of fixed layout; a step costs one host-to-device copy for the
-small tables and one per cache group for its page table.
+small tables and one per cache group for its page table, and the latter only when a
+page list has changed or other requests take part (rollout/cache.py:286-306).
 """
 from __future__ import annotations
 
@@ -116,6 +117,10 @@ class StepBuilder:
         # the staging buffer is written again only after the last step's copies have left it
         self._copied = torch.cuda.Event() if pin else None
         self._copy_pending = False
+        # the cache manager's page_key of the page tables that the device buffer holds: a step with
+        # the same key (no page list changed since, the same requests) finds them there
+        self._tables_on_device = None
+        self.page_table_copies = 0
 
     def _put(self, name: str, values) -> int:
         off, size = self._off[name]
@@ -163,7 +168,10 @@ class StepBuilder:
             self._put(f"slot_mapping{g}", gt.slot_mapping)
             self._put(f"cu_pages{g}", gt.cu_pages)
             self._put(f"kv_start{g}", gt.kv_start)
-            self._put(f"page_table{g}", gt.page_table)
+        tables_there = tables.page_key is not None and tables.page_key == self._tables_on_device
+        if not tables_there:
+            for g, gt in enumerate(tables.groups):
+                self._put(f"page_table{g}", gt.page_table)
         tiles = {}
         if pre:
             for rows in PREFILL_TILE_ROWS:
@@ -175,13 +183,15 @@ class StepBuilder:
         for g, gt in enumerate(tables.groups):
             off, _ = self._off[f"page_table{g}"]
             k = len(gt.page_table)
-            if k:
+            if k and not tables_there:
                 self._dev[off:off + k].copy_(self._host[off:off + k], non_blocking=True)
+                self.page_table_copies += 1
             n_pages = np.diff(gt.cu_pages).tolist()
             groups.append(GroupOnDevice(
                 self._view(f"slot_mapping{g}", T), self._view(f"page_table{g}", k),
                 self._view(f"cu_pages{g}", n + 1), self._view(f"kv_start{g}", n),
                 n_pages, max(n_pages) if n_pages else 0))
+        self._tables_on_device = tables.page_key
         if self._copied is not None:
             self._copied.record()
             self._copy_pending = True

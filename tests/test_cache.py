@@ -239,3 +239,62 @@ def test_a_pool_whose_head_rows_do_not_fit_32_bits_is_refused():
     with pytest.raises(ValueError, match="32 bits"):
         CacheManager({0: PagedKVSpec(8, 128)}, page_size=16, max_token=2 ** 28, max_requests=1, dtype=torch.bfloat16,
                      device="meta")
+
+
+def test_page_tables_are_copied_only_when_a_page_list_changed():
+    """100 decode steps of three requests: the page tables are put together and go to the device
+    again only in steps in which a request starts a new page or a window lets one go
+    (rollout/cache.py:286-306 skips its rebuild the same way); what the device buffer holds is right
+    in every step, also after other requests took part and in steps filled up for a graph."""
+    from return_amd.engine.batch import StepBuilder
+    P = 4
+
+    def check(cm, batch, ids):
+        for g in range(len(cm.groups)):
+            want = [p for rid in ids for p in cm.live[rid].pages[g]]
+            assert batch.groups[g].page_table.tolist()[:len(want)] == want
+            assert batch.groups[g].cu_pages.tolist()[:len(ids) + 1] == \
+                np.cumsum([0] + [len(cm.live[rid].pages[g]) for rid in ids]).tolist()
+            assert batch.groups[g].kv_start.tolist()[:len(ids)] == [cm.live[rid].first_pos[g] for rid in ids]
+
+    for window in (None, 6):
+        cm = manager(page=P, max_token=800, max_requests=4, window=window)
+        sb = StepBuilder(cm, 64, 4, "cpu")
+        prompts = {"a": 5, "b": 9, "c": 13}                # all one token into a page: they cross together
+        for rid in prompts:
+            cm.add_request(rid)
+        t = cm.begin_step(list(prompts.items()))
+        sb.build(t, [[0] * n for n in prompts.values()], [])
+        cm.end_step()
+        ids = list(prompts)
+        steps_that_copied = 0
+        version_at_last_tables = cm.version if window is None else None     # (a window may have let pages go)
+        for step in range(100):
+            copies, builds, version = sb.page_table_copies, cm.table_builds, cm.version
+            t = cm.begin_step([(r, 1) for r in ids])
+            batch = sb.build(t, [[0]] * 3, [0, 1, 2])
+            check(cm, batch, ids)
+            copied = sb.page_table_copies - copies
+            assert copied in (0, len(cm.groups))
+            assert (cm.table_builds - builds) == (1 if copied else 0)
+            # nothing changed since the last step's tables were made: nothing is made or copied
+            assert bool(copied) == (cm.version != version_at_last_tables)
+            version_at_last_tables = cm.version
+            steps_that_copied += bool(copied)
+            cm.end_step()
+        if window is None:
+            assert steps_that_copied == 25                 # every fourth
+        else:
+            assert 25 < steps_that_copied <= 51            # the window gives pages back in steps of its own
+        # other requests, then a filled-up step and its repeat
+        t = cm.begin_step([("a", 1), ("c", 1)])
+        check(cm, sb.build(t, [[0]] * 2, [0, 1]), ["a", "c"])
+        cm.end_step()
+        for _ in range(3):
+            t = cm.pad_tables(cm.begin_step([("a", 1), ("c", 1)]), 2)
+            batch = sb.build(t, [[0]] * 4, [0, 1, 2, 3])
+            check(cm, batch, ["a", "c"])
+            assert batch.groups[0].page_table.tolist()[-2:] == [cm.groups[0].spare_page] * 2
+            assert batch.groups[0].cu_pages.tolist()[-1] == len(batch.groups[0].page_table)
+            cm.end_step()
+        cm.check_invariants()
