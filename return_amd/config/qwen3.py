@@ -6,6 +6,11 @@ hidden // heads (rollout/monkey_patch/qwen3.py:117), num_key_value_heads
 (qwen3.py:17), rope inv_freq and attention_scaling (qwen3.py:121-127); it asserts
 that no layer has a sliding window (qwen3.py:130-132) and fuses gate and up only
 when there is no bias (qwen3.py:99-105).
+
+The rotation's base comes in one of two layouts: the key rope_theta at the top level (with
+rope_scaling beside it), or a dictionary rope_parameters {rope_theta, rope_type, ...}
+that newer config.json files carry instead. Both are read; one of them must give the base;
+any rope_type other than "default" is refused in either.
 """
 from __future__ import annotations
 
@@ -23,15 +28,34 @@ class Qwen3Config(ModelConfig):
     num_attention_heads: int
     intermediate_size: int
     max_position_embeddings: int
+    rms_norm_eps: float
+    rope_theta: float                              # top-level key, or rope_parameters.rope_theta
     num_key_value_heads: Optional[int] = None      # absent: one per query head
     head_dim: Optional[int] = None                 # absent: hidden_size // num_attention_heads
-    rms_norm_eps: float = 1e-6
-    rope_theta: float = 10000.0
     tie_word_embeddings: bool = False
     attention_bias: bool = False
     hidden_act: str = "silu"
     use_sliding_window: bool = False
     model_type: str = "qwen3"
+
+    @classmethod
+    def from_dict(cls, raw):
+        raw = dict(raw)
+        arch = (raw.get("architectures") or ["?"])[0]
+        params = raw.get("rope_parameters")
+        if params is not None:
+            if not isinstance(params, dict):
+                raise ConfigError(f"{arch}: rope_parameters must be a dictionary, got {params!r}")
+            kind = params.get("rope_type", params.get("type"))
+            if kind not in (None, "default"):
+                raise ConfigError(f"{arch}: rope_parameters {params!r} is not supported (only rope_type 'default')")
+            inner = params.get("rope_theta")
+            if inner is not None:
+                outer = raw.get("rope_theta")
+                if outer is not None and float(outer) != float(inner):
+                    raise ConfigError(f"{arch}: rope_theta is {outer!r} at the top level and {inner!r} in rope_parameters")
+                raw["rope_theta"] = inner
+        return super().from_dict(raw)
 
     def _coerce(self):
         super()._coerce()

@@ -21,8 +21,9 @@ import sys
 
 import numpy as np
 
-MAX_LIVE = 8            # request slots: traces keep up to four requests live, with room to spare
-ROUND_TO = 64           # a request's token count is rounded up to this for --max-tokens
+MAX_LIVE = 8            # default of --max-live: traces keep up to four requests live, with room to spare
+PAGE_SIZE = 16          # default of --page-size
+ROUND_TO = 64           # a request's token count is rounded up to this for --max-tokens (or to a larger page)
 
 
 def main(argv=None) -> int:
@@ -32,18 +33,28 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True, help="folder the logits are written to")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--page-size", type=int, default=PAGE_SIZE,
+                    help=f"tokens per cache page (default {PAGE_SIZE}): a divisor or a multiple of {ROUND_TO}; with "
+                         f"pages beyond {ROUND_TO} a request's count in --max-tokens is rounded up to whole pages")
+    ap.add_argument("--max-live", type=int, default=MAX_LIVE,
+                    help=f"most requests that are live at a time (default {MAX_LIVE})")
     args = ap.parse_args(argv)
+    page = args.page_size
+    if page < 1 or (ROUND_TO % page and page % ROUND_TO):
+        ap.error(f"--page-size {page}: must divide {ROUND_TO} or be a multiple of it")
+    if args.max_live < 1:
+        ap.error(f"--max-live {args.max_live}: at least one request")
 
     from ..config.engine import EngineConfig
     from .runner import ModelRunner, StepEntry
 
     os.makedirs(args.out, exist_ok=True)
-    page = 16                                   # divides ROUND_TO, so the pool is exactly max-tokens
-    pool = -(-args.max_tokens // ROUND_TO) * ROUND_TO
+    unit = max(page, ROUND_TO)                  # whole pages, so the pool is exactly max-tokens
+    pool = -(-args.max_tokens // unit) * unit
     # products by rule, not by the measurement at load, whose choices may differ from run to run:
     # two replays of a trace give the same bits
-    ec = EngineConfig(dtype=args.dtype, page_size=page, max_token=pool, max_reside=MAX_LIVE,
-                      max_step_tokens=max(pool, MAX_LIVE), prefill_chunk=pool, tune_products=False)
+    ec = EngineConfig(dtype=args.dtype, page_size=page, max_token=pool, max_reside=args.max_live,
+                      max_step_tokens=max(pool, args.max_live), prefill_chunk=pool, tune_products=False)
     runner = ModelRunner(args.model, engine_config=ec)
 
     for line in sys.stdin:

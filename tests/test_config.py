@@ -20,12 +20,37 @@ def test_reads_every_size_from_config_json():
 
 
 def test_defaults_of_optional_keys():
-    raw = {k: v for k, v in TINY_A.items() if k not in ("head_dim", "num_key_value_heads", "rms_norm_eps",
-                                                        "rope_theta", "tie_word_embeddings")}
+    raw = {k: v for k, v in TINY_A.items() if k not in ("head_dim", "num_key_value_heads", "tie_word_embeddings")}
     c = Qwen3Config.from_dict(raw)
     assert c.head_dim == 64 // 4                      # rollout/monkey_patch/qwen3.py:117
     assert c.num_key_value_heads == 4
-    assert c.rms_norm_eps == 1e-6 and c.rope_theta == 10000.0 and c.tie_word_embeddings is False
+    assert c.tie_word_embeddings is False
+
+
+def test_constants_of_the_model_have_no_stand_in():
+    """The norms' eps and the rotation's base are the model's own: a config.json without them is refused."""
+    for key in ("rms_norm_eps", "rope_theta"):
+        with pytest.raises(ConfigError, match=key):
+            Qwen3Config.from_dict({k: v for k, v in TINY_A.items() if k != key})
+
+
+def test_rotation_base_in_either_layout():
+    """rope_theta at the top level, or inside rope_parameters as newer config.json files have it; a
+    config.json of the second kind must not run with another base, and its rope_type is checked too."""
+    base = {k: v for k, v in TINY_B.items() if k != "rope_theta"}
+    new = Qwen3Config.from_dict(dict(base, rope_parameters={"rope_theta": 1000000.0, "rope_type": "default"}))
+    assert new.rope_theta == TINY_B["rope_theta"] == 1e6
+    assert new == Qwen3Config.from_dict(TINY_B)
+    both = Qwen3Config.from_dict(dict(TINY_B, rope_parameters={"rope_theta": 1e6, "rope_type": "default"}))
+    assert both.rope_theta == 1e6
+    with pytest.raises(ConfigError, match="rope_theta"):
+        Qwen3Config.from_dict(dict(TINY_B, rope_parameters={"rope_theta": 5e5}))          # two different bases
+    with pytest.raises(ConfigError, match="rope_theta"):
+        Qwen3Config.from_dict(dict(base, rope_parameters={"rope_type": "default"}))       # none at all
+    with pytest.raises(ConfigError, match="rope_parameters"):
+        Qwen3Config.from_dict(dict(base, rope_parameters={"rope_theta": 1e6, "rope_type": "yarn", "factor": 4.0}))
+    with pytest.raises(ConfigError, match="rope_parameters"):
+        Qwen3Config.from_dict(dict(base, rope_parameters="default"))
 
 
 def test_json_numbers_are_coerced():

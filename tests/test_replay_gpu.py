@@ -113,6 +113,27 @@ def test_trace_run_program(folder_a, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program_at_the_page_size_of_tiny_b(folder_b, tmp_path, dtype):
+    """Tiny B at its own geometry (pages of 32 rows) and with exactly as many request slots as the
+    trace has live requests at a time, both given on the command line."""
+    reqs = requests_for(TINY_B["vocab_size"], TINY_B["max_position_embeddings"])
+    want = oracle(folder_b, reqs)
+    steps = tt.mixed(reqs, seed=5)
+    got = tt.run_program(folder_b, dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps),
+                         TINY_B["vocab_size"], extra=("--page-size", "32", "--max-live", "4"))
+    compare(got, want, reqs, dtype)
+
+
+def test_trace_run_program_refuses_a_page_size_it_cannot_count_in(folder_a, tmp_path):
+    import subprocess
+    import sys
+    p = subprocess.run([sys.executable, tt.os.path.join(tt.ROOT, "bin", "trace_run"), "--model", folder_a, "--dtype",
+                        "float32", "--out", str(tmp_path), "--max-tokens", "64", "--page-size", "24"],
+                       stdin=subprocess.DEVNULL, capture_output=True, text=True)
+    assert p.returncode == 2 and "--page-size 24" in p.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folder_b, dtype):
     """300 tokens one by one after a short prompt."""
     toks = tt.random_tokens(TINY_B["vocab_size"], 320, seed=77)

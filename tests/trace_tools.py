@@ -130,10 +130,10 @@ def run_in_process(runner, steps):
     return got
 
 
-def run_program(model_dir, dtype, steps, out_dir, max_tokens, vocab, env=None):
+def run_program(model_dir, dtype, steps, out_dir, max_tokens, vocab, env=None, extra=()):
     """Drive bin/trace_run as a child process; same result shape as run_in_process."""
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
-           "--out", out_dir, "--max-tokens", str(max_tokens)]
+           "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
     p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
     got, pos = {}, {}
     for s in steps:
