@@ -69,8 +69,6 @@ class StepBatch:
     prefill_tiles: dict = dataclasses.field(default_factory=dict)
 
 
-PREFILL_TILE_ROWS = (64, 128)      # query rows per workgroup of the prefill attention kernel, by head size
-
 
 def prefill_tiles(q_lens, q_starts=None, rows=64):
     """(request number, first row) of every tile of ``rows`` rows, for requests with more than
@@ -84,8 +82,11 @@ def prefill_tiles(q_lens, q_starts=None, rows=64):
 class StepBuilder:
     """Fixed device buffers for the tables of a step, sized for the worst case."""
 
-    def __init__(self, cache: CacheManager, max_step_tokens: int, max_requests: int, device):
+    def __init__(self, cache: CacheManager, max_step_tokens: int, max_requests: int, device, tile_rows=()):
+        """tile_rows: heights of the q tiles that the model's mixers want listed for the requests that
+        bring more than one token (what their attention kernels' grids run over); none: no lists."""
         self.cache = cache
+        self.tile_rows = tuple(sorted(int(r) for r in tile_rows))
         self.device = torch.device(device)
         self.max_tokens = int(max_step_tokens)
         self.max_requests = int(max_requests)
@@ -93,7 +94,7 @@ class StepBuilder:
         layout = [("token_ids", T), ("positions", T), ("logit_rows", T), ("cu_q", N + 1),
                   ("q_start", N), ("seq_lens", N), ("slot_ids", N), ("decode_segs", N),
                   ("prefill_toks", T)]
-        layout += [(f"prefill_tiles{rows}", 2 * (T // rows + N)) for rows in PREFILL_TILE_ROWS]
+        layout += [(f"prefill_tiles{rows}", 2 * (T // rows + N)) for rows in self.tile_rows]
         for g in range(G):
             layout += [(f"slot_mapping{g}", T), (f"cu_pages{g}", N + 1), (f"kv_start{g}", N)]
         self._small_end = None
@@ -174,7 +175,7 @@ class StepBuilder:
                 self._put(f"page_table{g}", gt.page_table)
         tiles = {}
         if pre:
-            for rows in PREFILL_TILE_ROWS:
+            for rows in self.tile_rows:
                 tiles[rows] = prefill_tiles(tables.q_lens, tables.q_start, rows)
                 self._put(f"prefill_tiles{rows}", np.asarray(tiles[rows], dtype=np.int32).reshape(-1))
         # one copy for the small tables, one per group for the used part of its page table

@@ -61,7 +61,8 @@ class ModelRunner:
         self._check_cache_fits()
         self.cache = CacheManager(self.model.cache_layers(), ec.page_size, ec.max_token,
                                   ec.max_reside, self.rt.dtype, self.rt.device)
-        self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device)
+        self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device,
+                                   tile_rows=self.model.step_needs()["prefill_tile_rows"])
         self.vocab_size = self.spec.vocab_size
         self.max_position = self.spec.max_position
         # decode-only steps replayed from captured HIP graphs (rollout/model.py:346-407 captures one
@@ -253,6 +254,10 @@ class ModelRunner:
         graphs = self.engine_config.use_graphs and self.rt.device.type == "cuda"
         rows = self.graph_batch_size(n) if graphs else n
         pad = rows - n
+        if graphs:
+            key = self._graph_key(rows, max(self.cache.seq_len(rid) for rid in request_ids) + 1)
+            if key not in self._graphs:
+                self._capture(key)
         tables = self.cache.begin_step([(rid, 1) for rid in request_ids])
         try:
             tables = self.cache.pad_tables(tables, pad)
@@ -270,7 +275,7 @@ class ModelRunner:
                                list(top_p) + [1.0] * pad, list(uniforms) + [0.0] * pad)
             with torch.no_grad():
                 if graphs:
-                    logits, picked = self._replay(batch)
+                    logits, picked = self._replay(key)
                 else:
                     logits, picked = self._decode_body(batch)
         finally:
@@ -300,31 +305,46 @@ class ModelRunner:
             return n
         return min(-(-n // 8) * 8, max(n, self.engine_config.max_reside))
 
-    def _replay(self, batch):
+    def _graph_key(self, rows: int, longest: int):
+        """(batch size, context bucket) of the graph that serves `rows` decoding rows whose longest
+        request holds `longest` tokens after the step."""
         bucket = 256
-        while bucket < batch.max_decode_seq_len:
+        while bucket < longest:
             bucket *= 2
-        key = (batch.n_seqs, bucket)
-        entry = self._graphs.get(key)
-        batch.max_decode_seq_len = bucket        # grid and scratch sizes cover the whole bucket
-        batch.decode_len_is_bound = True
-        if entry is None:
-            # what a launch derives from the context length (grid, split size, scratch) now
-            # derives from the bucket, and so holds for every replay
-            side = torch.cuda.Stream(self.rt.device)
-            side.wait_stream(torch.cuda.current_stream(self.rt.device))
-            with torch.cuda.stream(side):
-                self._decode_body(batch)                      # warm-up outside the capture
-            torch.cuda.current_stream(self.rt.device).wait_stream(side)
-            torch.cuda.synchronize(self.rt.device)
-            graph = torch.cuda.CUDAGraph()
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits, picked = self._decode_body(batch)
-            entry = (graph, logits, picked)
-            self._graphs[key] = entry
-        graph, logits, picked = entry
+        return rows, bucket
+
+    def _capture(self, key) -> None:
+        """Warms the decode step up and captures it for one (batch size, context bucket), on rows that
+        belong to no request: every row sits on the spare page and the spare state slot. A step is
+        not idempotent in general (a mixer with state of fixed size advances it), so nothing that a
+        request holds may be touched by the warm-up; the first real step of this shape is a replay
+        like every later one. What a launch derives from the context length (grid, split size,
+        scratch) derives from the bucket here, and so holds for every replay."""
+        rows, bucket = key
+        dev = self.rt.device
+        tables = self.cache.pad_tables(self.cache.begin_step([]), rows)
+        try:
+            batch = self.builder.build(tables, [[0]] * rows, list(range(rows)))
+            batch.max_decode_seq_len = bucket
+            batch.decode_len_is_bound = True
+            with torch.no_grad():
+                side = torch.cuda.Stream(dev)
+                side.wait_stream(torch.cuda.current_stream(dev))
+                with torch.cuda.stream(side):
+                    self._decode_body(batch)                      # warm-up outside the capture
+                torch.cuda.current_stream(dev).wait_stream(side)
+                torch.cuda.synchronize(dev)
+                graph = torch.cuda.CUDAGraph()
+                if self._graph_pool is None:
+                    self._graph_pool = torch.cuda.graph_pool_handle()
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    logits, picked = self._decode_body(batch)
+        finally:
+            self.cache.end_step()
+        self._graphs[key] = (graph, logits, picked)
+
+    def _replay(self, key):
+        graph, logits, picked = self._graphs[key]
         graph.replay()
         return logits, picked
 

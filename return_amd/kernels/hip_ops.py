@@ -520,6 +520,23 @@ class HipOps:
         return best / launches
 
     # ------------------------------------------------------------------ attention
+    MAX_HEAD_DIM = 512
+
+    def check_attention_sizes(self, n_q, n_kv, D, dtype):
+        """Raises for head counts and sizes that no attention kernel here takes (asked when a model is built)."""
+        if D > self.MAX_HEAD_DIM or D < 1:
+            raise KernelError(f"attention: head size {D} is beyond the kernels' {self.MAX_HEAD_DIM}")
+        if n_kv < 1 or n_q % n_kv:
+            raise KernelError(f"attention: {n_q} query heads over {n_kv} kv heads")
+        _code(dtype)
+
+    def prefill_tile_rows(self, D, dtype):
+        """Rows per q tile of the list that attention() reads from step.prefill_tiles for requests with
+        more than one token, or None where the kernel that serves this head size takes no list."""
+        if dtype == torch.bfloat16 and D % 16 == 0 and D <= 256:
+            return int(self.lib.ra_attention_prefill_tile_rows(D))
+        return None
+
     def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
         self._want(q, "q", dims=3)
         self._want(out, "attention output", q.dtype, 3)
@@ -531,8 +548,7 @@ class HipOps:
             raise KernelError(f"attention: q {tuple(q.shape)}, out {tuple(out.shape)}, step of {step.n_tokens}")
         if n_q % n_kv:
             raise KernelError(f"attention: {n_q} query heads over {n_kv} kv heads")
-        if D > 512:
-            raise KernelError(f"attention: head size {D} is beyond the kernel's 512")
+        self.check_attention_sizes(n_q, n_kv, D, q.dtype)
         P = k_pool.shape[2]
         window = int(window)
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))

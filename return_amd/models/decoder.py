@@ -25,12 +25,17 @@ class Decoder:
 
         build = lambda cat, ps, shared=None: part_class(cat, ps.kind)(ps.params, tensors_of(ps), rt, shared)
         self.positions = {name: build("position", ps) for name, ps in spec.positions.items()}
-        self.embedding = build("embedding", spec.embedding)
+        self.embedding = build("embedding", spec.embedding, self.positions)
         self.blocks = []
         for b in spec.blocks:
             if b.arrangement not in BLOCKS:
                 raise KeyError(f"no block arrangement {b.arrangement!r}; registered: {sorted(BLOCKS)}")
-            self.blocks.append(BLOCKS[b.arrangement](b, tensors_of, rt, self.positions))
+
+            def build_named(name, b=b):
+                b.part(name)                              # (a clear error for a name the block lacks)
+                category, ps = b.parts[name]
+                return build(category, ps, self.positions)
+            self.blocks.append(BLOCKS[b.arrangement](b, build_named))
         self.final_norm = build("norm", spec.final_norm)
         self.head = build("head", spec.head)
         self.schedule = list(spec.schedule)
@@ -45,7 +50,7 @@ class Decoder:
         for call in self.schedule:
             if call.cache is None:
                 continue
-            spec = self.blocks[call.block].mixer.cache_spec()
+            spec = self.blocks[call.block].cache_spec()
             if spec is None:
                 raise ValueError(f"block {call.block} keeps nothing but the run order gives it cache layer {call.cache}")
             if call.cache in need and need[call.cache] != spec:
@@ -60,9 +65,18 @@ class Decoder:
             raise ValueError(f"cache layers {sorted(missing)} are read but never written")
         return need
 
+    def step_needs(self):
+        """What the parts ask of a step's tables beyond what every step has, merged over the model:
+        {"prefill_tile_rows": set of q-tile heights whose tile lists the attention kernels read}."""
+        tile_rows = set()
+        for block in self.blocks:
+            needs = block.step_needs() if hasattr(block, "step_needs") else {}
+            tile_rows.update(needs.get("prefill_tile_rows", ()))
+        return {"prefill_tile_rows": tile_rows}
+
     def forward(self, step, cache):
         """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
-        h = self.embedding.forward(step.token_ids)
+        h = self.embedding.forward(step.token_ids, step)
         pending = None
         for call in self.schedule:
             view = cache.view(call.cache) if call.cache is not None else None

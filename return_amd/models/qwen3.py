@@ -32,8 +32,8 @@ def build_spec(cfg: Qwen3Config) -> ModelSpec:
             "swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size},
             {"gate_proj": p + "mlp.gate_proj.weight", "up_proj": p + "mlp.up_proj.weight",
              "down_proj": p + "mlp.down_proj.weight"})
-        blocks.append(BlockSpec(attn, mlp, norm(p + "input_layernorm.weight"),
-                                norm(p + "post_attention_layernorm.weight"), "pre_norm"))
+        blocks.append(BlockSpec.pre_norm(attn, mlp, norm(p + "input_layernorm.weight"),
+                                         norm(p + "post_attention_layernorm.weight")))
     tied = cfg.tie_word_embeddings
     return ModelSpec(
         architecture=cfg.architecture, hidden_size=H, vocab_size=cfg.vocab_size,

@@ -44,6 +44,8 @@ class PagedAttention:
         self.d = int(params["head_dim"])
         if self.n_q % self.n_kv:
             raise ValueError(f"{self.n_q} query heads are not a multiple of {self.n_kv} kv heads")
+        if hasattr(rt.ops, "check_attention_sizes"):      # sizes the kernels do not take are refused now, not at the first step
+            rt.ops.check_attention_sizes(self.n_q, self.n_kv, self.d, rt.dtype)
         self.scale = float(params["scale"]) if params.get("scale") is not None else self.d ** -0.5
         self.window = params.get("window")
         self.eps = params.get("qk_norm_eps")
@@ -59,6 +61,12 @@ class PagedAttention:
 
     def cache_spec(self):
         return PagedKVSpec(self.n_kv, self.d, self.window)
+
+    def step_needs(self):
+        """The q-tile list that the kernel set's attention reads for requests with more than one token."""
+        ops = self.rt.ops
+        rows = ops.prefill_tile_rows(self.d, self.rt.dtype) if hasattr(ops, "prefill_tile_rows") else None
+        return {"prefill_tile_rows": {rows}} if rows else {}
 
     def forward(self, x, step, cache, write_cache=True):
         rt, ops = self.rt, self.rt.ops

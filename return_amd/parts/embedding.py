@@ -23,8 +23,9 @@ class TokenEmbedding:
         self.hidden = int(params["hidden_size"])
         self.table = rt.matrix(tensors["weight"])
 
-    def forward(self, token_ids):
-        """int32 ids [T] -> fp32 residual stream [T, H]."""
+    def forward(self, token_ids, step=None):
+        """int32 ids [T] -> fp32 residual stream [T, H]. (step: the whole step, for an embedding that
+        adds something of the positions; this one does not look at it.)"""
         h = self.rt.empty(token_ids.shape[0], self.hidden, dtype=torch.float32)
         self.rt.ops.embed(self.table, token_ids, h)
         return h

@@ -8,7 +8,7 @@ schedule. No part knows which model it is in.
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 
 @dataclasses.dataclass
@@ -21,15 +21,30 @@ class PartSpec:
 
 @dataclasses.dataclass
 class BlockSpec:
-    """One layer: a mixer and a feed-forward, each behind a norm, and how they are arranged.
+    """One layer: its parts by name, and the arrangement (a class registered with
+    return_amd.parts.block.register_arrangement) that builds and runs them.
 
-    arrangement "pre_norm":  h += mixer(mixer_norm(h));  h += feed_forward(feed_forward_norm(h))
+    parts: name -> (category, PartSpec). Which names there are is the arrangement's business:
+    "pre_norm" has mixer_norm, mixer, feed_forward_norm and feed_forward
+    (h += mixer(mixer_norm(h)); h += feed_forward(feed_forward_norm(h))); another arrangement
+    may have post-norms, no feed-forward or two mixers. Tensor names, shapes and random
+    weights follow from the parts, whatever their names.
     """
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Dict[str, Tuple[str, PartSpec]]
     arrangement: str = "pre_norm"
+
+    @classmethod
+    def pre_norm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
+                 feed_forward_norm: PartSpec) -> "BlockSpec":
+        return cls({"mixer_norm": ("norm", mixer_norm), "mixer": ("mixer", mixer),
+                    "feed_forward_norm": ("norm", feed_forward_norm),
+                    "feed_forward": ("feed_forward", feed_forward)}, "pre_norm")
+
+    def part(self, name: str) -> PartSpec:
+        if name not in self.parts:
+            raise KeyError(f"arrangement {self.arrangement!r} wants a part named {name!r}; the block has "
+                           f"{sorted(self.parts)}")
+        return self.parts[name][1]
 
 
 @dataclasses.dataclass
@@ -66,10 +81,8 @@ class ModelSpec:
         for name, p in self.positions.items():
             yield "position", f"positions[{name}]", p
         for i, b in enumerate(self.blocks):
-            yield "norm", f"blocks[{i}].mixer_norm", b.mixer_norm
-            yield "mixer", f"blocks[{i}].mixer", b.mixer
-            yield "norm", f"blocks[{i}].feed_forward_norm", b.feed_forward_norm
-            yield "feed_forward", f"blocks[{i}].feed_forward", b.feed_forward
+            for name, (category, p) in b.parts.items():
+                yield category, f"blocks[{i}].{name}", p
         yield "norm", "final_norm", self.final_norm
         yield "head", "head", self.head
 

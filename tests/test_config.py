@@ -114,10 +114,10 @@ def test_spec_follows_the_configuration():
         cfg = Qwen3Config.from_dict(raw)
         spec = build_spec(cfg)
         assert len(spec.blocks) == cfg.num_hidden_layers == len(spec.schedule)
-        m = spec.blocks[0].mixer.params
+        m = spec.blocks[0].part("mixer").params
         assert (m["num_heads"], m["num_kv_heads"], m["head_dim"]) == (
             cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim)
-        assert spec.blocks[0].mixer_norm.params["eps"] == cfg.rms_norm_eps
+        assert spec.blocks[0].part("mixer_norm").params["eps"] == cfg.rms_norm_eps
         assert spec.positions["rotary"].params["theta"] == cfg.rope_theta
         tied = spec.head.tensors["weight"] == spec.embedding.tensors["weight"]
         assert tied == cfg.tie_word_embeddings

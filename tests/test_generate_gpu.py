@@ -135,6 +135,48 @@ def test_kept_sessions_on_the_gpu(folder_b, dtype):
     assert not eng.runner.cache.live and all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
 
 
+@pytest.mark.parametrize("lookahead", [True, False])
+def test_kept_sessions_that_end_on_a_stop_sequence_found_a_step_late(folder_b, lookahead):
+    """Kept sessions, stop sequences, graphs and steps launched ahead together, over three turns: with
+    steps launched ahead a stop sequence is found when the next step, which feeds the last token back,
+    is already under way, so the kept cache holds one token more than without; the next turn repeats
+    the conversation and must find every one of them right. 32-bit: the answers are the plain
+    implementation's, cut after the stop sequence."""
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    cfg, w = plain.read_folder(folder_b)
+    V = TINY_B["vocab_size"]
+    eng = Engine(folder_b, dtype="float32", page_size=16, max_token=2048, max_reside=4, max_step_tokens=64,
+                 prefill_chunk=32, use_graphs=True, lookahead=lookahead, tune_products=False)
+    convs = {k: tt.random_tokens(V, n, seed=90 + n) for k, n in (("a", 6), ("b", 31), ("c", 70), ("d", 16))}
+    stop_after = {"a": 3, "b": 9, "c": 1, "d": None}           # d runs to its length
+    for turn in range(3):
+        ids = list(convs)
+        free = {k: plain.greedy_generate(cfg, w, convs[k], 12) for k in ids}
+        params, want = [], {}
+        for k in ids:
+            n = stop_after[k]
+            if n is None:
+                params.append(SamplingParams(temperature=0.0, max_new_tokens=12))
+                want[k] = (free[k], "length")
+                continue
+            stop = free[k][n:n + 2]
+            first = next(i for i in range(1, 12) if free[k][i - 1:i + 1] == stop)      # (it may come earlier by chance)
+            params.append(SamplingParams(temperature=0.0, max_new_tokens=12, stop_ids=[stop]))
+            want[k] = (free[k][:first + 1], "stop")
+        out = eng.generate([convs[k] for k in ids], params, session_ids=ids, keep=turn < 2)
+        for k, r in zip(ids, out):
+            assert (r.output_ids, r.finish_reason) == want[k], (turn, k)
+            assert (r.cached_tokens > 0) == (turn > 0) and r.cached_tokens < len(convs[k])
+            if turn > 0:
+                assert r.cached_tokens >= held[k] - 1           # all but at most the last token fed back
+            convs[k] = convs[k] + r.output_ids + tt.random_tokens(V, 2 + turn, seed=turn * 7 + len(convs[k]))
+        held = {k: eng.runner.cache.seq_len(k) for k in ids} if turn < 2 else {}
+        eng.runner.cache.check_invariants()
+    assert eng.runner._graphs
+    assert not eng.runner.cache.live and all(g.pages.in_use() == 0 for g in eng.runner.cache.groups)
+
+
 def test_command_line_turns_of_a_session(folder_a, tmp_path):
     """A session_id that comes again is the session's next turn: its cache was kept for it."""
     cfg, w = plain.read_folder(folder_a)

@@ -104,7 +104,10 @@ def test_head_rmsnorm_and_rope(ops, ref, dtype, D):
                                            (3, 1, 80, 32, False), (8, 2, 128, 128, True),
                                            (2, 2, 256, 64, True), (1, 1, 512, 512, True),
                                            (7, 1, 80, 80, True), (2, 1, 192, 192, False), (3, 1, 64, 0, True),
-                                           (9, 3, 256, 256, True)])
+                                           (9, 3, 256, 256, True),
+                                           # head sizes that are no multiple of 16, or beyond 256: the general kernel
+                                           (3, 1, 24, 24, True), (4, 2, 40, 40, True), (5, 1, 72, 36, True),
+                                           (2, 1, 320, 320, True), (3, 3, 6, 6, True), (2, 2, 130, 130, False)])
 def test_qkv_prepare(ops, ref, dtype, Hq, Hkv, D, R, norm):
     T, P, pages = 11, 8, 6
     qkv = rnd(T, (Hq + 2 * Hkv) * D, dtype=dtype, seed=11)
@@ -401,10 +404,10 @@ def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
                  n_prefill_tokens=cu_q[-1] - len(dec),
                  prefill_toks=i32([t for i in pre for t in range(cu_q[i], cu_q[i + 1])]) if both else None,
                  prefill_segs=pre)
-    from return_amd.engine.batch import PREFILL_TILE_ROWS, prefill_tiles
+    from return_amd.engine.batch import prefill_tiles
     extra.update(prefill_tiles={})
     if any(q != 1 for q in q_lens):
-        extra.update(prefill_tiles={rows: i32(prefill_tiles(q_lens, q_starts, rows)) for rows in PREFILL_TILE_ROWS})
+        extra.update(prefill_tiles={rows: i32(prefill_tiles(q_lens, q_starts, rows)) for rows in (64, 128)})
     return types.SimpleNamespace(**extra, n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
                                  seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
                                  q_lens=list(q_lens), q_starts=list(q_starts),
@@ -431,6 +434,13 @@ ATTN_CASES = [
     (24, 1, 64, 16, [(1, 100)], 0),
     (40, 2, 128, 16, [(1, 300), (9, 20), (1, 64), (1, 0)], 0),     # 20 heads a kv head: two waves of 16 and 4
     (33, 1, 48, 8, [(1, 77), (1, 200)], 50),
+    # head sizes that the MFMA kernels do not take (no multiple of 16, or beyond 256): the plain kernel in both precisions
+    (6, 2, 24, 16, [(1, 130), (20, 7), (1, 0), (70, 64)], 0),
+    (5, 1, 40, 8, [(1, 300), (33, 0), (1, 17)], 0),
+    (4, 4, 72, 16, [(9, 20), (1, 200), (1, 1)], 25),
+    (4, 2, 320, 16, [(1, 150), (40, 3), (2, 62)], 0),
+    (3, 1, 6, 4, [(1, 99), (17, 0)], 0),
+    (2, 1, 512, 16, [(1, 70), (5, 30)], 0),
 ]
 
 

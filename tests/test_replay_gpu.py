@@ -171,6 +171,8 @@ ODD = [
     (16, 60, 3, 96, 328, 1000, 2, 8, True),       # 20 query heads to a kv head: two waves of the decode kernel
     (80, 7, 1, 100, 48, 1000, 1, 32, False),      # 7 heads on one kv head, head size 80
     (256, 5, 5, 136, 100, 97, 2, 48, False),      # the largest head size, a page of 48
+    (40, 6, 2, 96, 72, 331, 2, 16, True),         # a head size that is no multiple of 16: the plain attention, in bfloat16 too
+    (320, 2, 1, 64, 48, 97, 1, 8, False),         # a head size beyond the MFMA kernels' 256
 ]
 
 

@@ -3,7 +3,10 @@ registries only, with
   - a mixer that keeps state of its own (an exponential moving average per request),
   - a feed-forward with routing (top-1 of two experts, router logits in 32-bit),
   - a position encoding that is no rotation (keys scaled by their position),
+  - an embedding that adds a learned vector per absolute position (it sees the step's positions),
   - a windowed attention layer (pages of its own, given back as the window passes),
+  - a block arrangement with other parts than the framework's own (no feed-forward, a norm after
+    the mixer as well as before it),
   - a run order that calls one block twice and lets one layer read another layer's cache.
 It is built and stepped without a change to the framework's files and compared, in 32-bit,
 with a dense whole-sequence evaluation written below. This toy is no model of anyone's."""
@@ -16,6 +19,7 @@ from return_amd.cache.spec import StateSpec
 from return_amd.config import EngineConfig, ModelConfig, register_architecture
 from return_amd.engine import ModelRunner
 from return_amd.parts import BlockSpec, LayerCall, ModelSpec, PartSpec, register_part
+from return_amd.parts.block import register_arrangement
 from return_amd.weights import random_weights
 from tests import trace_tools as tt
 from tests.plain import qwen3_plain as plain
@@ -42,6 +46,13 @@ class EmaMixer:
 
     def forward(self, x, step, cache, write_cache=True):
         u = self.rt.ops.linear(x, self.w).float()
+        if step.all_decode:
+            # one token each: everything on the device from the step's tables, no number of the host's
+            # is baked in, so the step can be captured in a graph and replayed on other requests
+            state = cache.tensors["s"]
+            s = self.decay * state.index_select(0, step.slot_ids) + u
+            state.index_copy_(0, step.slot_ids.long(), s)
+            return s.to(x.dtype)
         y = torch.empty_like(u)
         for i in range(step.n_seqs):
             a, b = step.cu_q_host[i], step.cu_q_host[i + 1]
@@ -77,6 +88,14 @@ class RoutedFeedForward:
 
     def forward(self, x, step=None):
         choice = (x.float() @ self.router.t()).argmax(-1)
+        if step is not None and step.all_decode:
+            # few rows: every expert on every row and a choice on the device (nothing waits for the
+            # device, so the step can be captured in a graph)
+            y = torch.zeros_like(x)
+            for e in range(self.E):
+                out = self.rt.ops.linear(self.rt.ops.linear(x, self.w1[e]).relu().contiguous(), self.w2[e])
+                y = torch.where((choice == e)[:, None], out, y)
+            return y
         y = torch.zeros_like(x)
         for e in range(self.E):
             rows = (choice == e).nonzero().flatten()
@@ -102,7 +121,44 @@ class KeyFade:
             k.mul_((1.0 / (1.0 + positions.float() / self.horizon)).to(k.dtype)[:, None, None])
 
 
+class PositionedEmbedding:
+    """table[token] + place[position]: an absolute position encoding, added where the tokens come in."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        return {"table": (params["vocab_size"], params["hidden_size"]),
+                "place": (params["max_position"], params["hidden_size"])}
+
+    @staticmethod
+    def random_init(params, role):
+        return "embedding"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.table = tensors["table"].to(rt.device).float()
+        self.place = tensors["place"].to(rt.device).float()
+
+    def forward(self, token_ids, step):
+        return (self.table.index_select(0, token_ids) + self.place.index_select(0, step.positions)).contiguous()
+
+
+class MixerBetweenNorms:
+    """h += after(mixer(before(h))): three parts, none of them a feed-forward."""
+
+    def __init__(self, spec, build):
+        self.before, self.mixer, self.after = build("before"), build("mixer"), build("after")
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def forward(self, h, pending, step, cache, write_cache=True):
+        x = self.before.forward(h, pending)
+        a = self.mixer.forward(x, step, cache, write_cache)
+        return h, self.after.forward(a.float().contiguous())
+
+
 register_part("mixer", "toy_ema", EmaMixer)
+register_part("embedding", "toy_positioned", PositionedEmbedding)
+register_arrangement("toy_mixer_between_norms", MixerBetweenNorms)
 register_part("feed_forward", "toy_routed", RoutedFeedForward)
 register_part("position", "toy_key_fade", KeyFade)
 
@@ -143,18 +199,24 @@ def toy_spec(c: ToyConfig) -> ModelSpec:
                       dict([("router", "blocks.1.ffn.router")] +
                            [(f"w{k}_{e}", f"blocks.1.ffn.w{k}_{e}") for k in (1, 2) for e in (0, 1)]))
     blocks = [
-        BlockSpec(attn(0, None, "rotary", c.eps), mlp(0), norm("blocks.0.n1"), norm("blocks.0.n2")),
-        BlockSpec(PartSpec("toy_ema", {"hidden_size": H, "decay": c.decay}, {"w": "blocks.1.ema.w"}), routed,
-                  norm("blocks.1.n1"), norm("blocks.1.n2")),
-        BlockSpec(attn(2, c.window, "fade", None), mlp(2), norm("blocks.2.n1"), norm("blocks.2.n2")),
-        BlockSpec(attn(3, None, "rotary", c.eps), mlp(3), norm("blocks.3.n1"), norm("blocks.3.n2")),
+        BlockSpec.pre_norm(attn(0, None, "rotary", c.eps), mlp(0), norm("blocks.0.n1"), norm("blocks.0.n2")),
+        BlockSpec.pre_norm(PartSpec("toy_ema", {"hidden_size": H, "decay": c.decay}, {"w": "blocks.1.ema.w"}), routed,
+                           norm("blocks.1.n1"), norm("blocks.1.n2")),
+        BlockSpec.pre_norm(attn(2, c.window, "fade", None), mlp(2), norm("blocks.2.n1"), norm("blocks.2.n2")),
+        BlockSpec.pre_norm(attn(3, None, "rotary", c.eps), mlp(3), norm("blocks.3.n1"), norm("blocks.3.n2")),
+        BlockSpec({"before": ("norm", norm("blocks.4.before")),
+                   "mixer": ("mixer", PartSpec("toy_ema", {"hidden_size": H, "decay": 0.5}, {"w": "blocks.4.ema.w"})),
+                   "after": ("norm", norm("blocks.4.after"))}, "toy_mixer_between_norms"),
     ]
     schedule = [LayerCall(0, cache=0), LayerCall(1, cache=1), LayerCall(2, cache=2),
                 LayerCall(0, cache=3),                           # block 0 a second time, a cache of its own
-                LayerCall(3, cache=0, writes_cache=False)]       # block 3 reads what the first call wrote
+                LayerCall(3, cache=0, writes_cache=False),       # block 3 reads what the first call wrote
+                LayerCall(4, cache=4)]
     return ModelSpec(
         architecture=c.architecture, hidden_size=H, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
-        embedding=PartSpec("token_embedding", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "embed"}),
+        embedding=PartSpec("toy_positioned", {"vocab_size": c.vocab_size, "hidden_size": H,
+                                              "max_position": c.max_position_embeddings},
+                           {"table": "embed", "place": "embed_place"}),
         positions={"rotary": PartSpec("rotary", {"head_dim": c.head_dim, "rotary_dim": c.head_dim // 2,
                                                  "theta": 500.0, "max_position": c.max_position_embeddings}),
                    "fade": PartSpec("toy_key_fade", {"horizon": 40.0})},
@@ -172,7 +234,7 @@ TOY = dict(architectures=["ToyForTests"], vocab_size=97, hidden_size=48, heads=4
 def toy_plain_logits(c, w, tokens):
     T, D = len(tokens), c.head_dim
     pos = torch.arange(T)
-    h = w["embed"][torch.tensor(tokens)]
+    h = w["embed"][torch.tensor(tokens)] + w["embed_place"][:T]
     kv0 = {}
 
     def attention(x, i, window, kind, qk_eps, keep=None, reuse=None):
@@ -222,6 +284,11 @@ def toy_plain_logits(c, w, tokens):
     h = block0(h, None)
     h = h + attention(plain.rms_norm(h, w["blocks.3.n1"], c.eps), 3, None, "rotary", c.eps, reuse="first")
     h = h + swiglu(plain.rms_norm(h, w["blocks.3.n2"], c.eps), 3)
+    u, s, ys = plain.rms_norm(h, w["blocks.4.before"], c.eps) @ w["blocks.4.ema.w"].T, torch.zeros(c.hidden_size), []
+    for t in range(T):
+        s = 0.5 * s + u[t]
+        ys.append(s)
+    h = h + plain.rms_norm(torch.stack(ys), w["blocks.4.after"], c.eps)
     return plain.rms_norm(h, w["final_norm"], c.eps) @ w["head"].T
 
 
@@ -239,7 +306,7 @@ def run_toy(device, ops):
         runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()},
                              engine_config=ec, ops=ops)
         cache = runner.cache
-        assert len(cache.groups) == 2 and len(cache.state_layers) == 1      # full, windowed; one state layer
+        assert len(cache.groups) == 2 and len(cache.state_layers) == 2      # full, windowed; two state layers
         got = tt.run_in_process(runner, steps)
         for rid, toks in reqs.items():
             for p in range(len(toks)):
@@ -257,3 +324,41 @@ def test_toy_architecture_on_cpu_stand_in():
 @pytest.mark.gpu
 def test_toy_architecture_on_gpu():
     run_toy("cuda:0", None)
+
+
+def generate_toy(device, ops, **options):
+    """Greedy generation of the toy through Engine.generate against the dense evaluation: the state
+    of the toy's mixers advances once per token, whichever way the engine runs its decode steps."""
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    cfg = ToyConfig.from_dict(TOY)
+    weights = random_weights(toy_spec(cfg), seed=4, std=0.08, norm_jitter=0.05, dtype="float32")
+    prompts = [tt.random_tokens(cfg.vocab_size, n, seed=70 + n) for n in (9, 1, 30, 17, 4)]
+    new = 24
+    want = []
+    for p in prompts:
+        toks = list(p)
+        for _ in range(new):
+            toks.append(int(toy_plain_logits(cfg, weights, toks)[-1].argmax()))
+        want.append(toks[len(p):])
+    ec = EngineConfig(dtype="float32", page_size=4, max_token=512, max_reside=3, max_step_tokens=32,
+                      prefill_chunk=16, device=device, **options)
+    runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()}, engine_config=ec, ops=ops)
+    got = Engine(runner=runner).generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=new))
+    assert [r.output_ids for r in got] == want
+    return runner
+
+
+def test_toy_generation_on_cpu_stand_in():
+    from tests.torch_ops import TorchOps
+    generate_toy("cpu", TorchOps(), lookahead=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("use_graphs", [True, False])
+@pytest.mark.parametrize("lookahead", [True, False])
+def test_toy_generation_on_gpu(use_graphs, lookahead):
+    """With graphs, the warm-up and the capture of every new (batch size, context bucket) must leave the
+    requests' state alone: a step that ran twice would advance the moving averages twice."""
+    runner = generate_toy("cuda:0", None, use_graphs=use_graphs, lookahead=lookahead)
+    assert bool(runner._graphs) == use_graphs
