@@ -103,9 +103,9 @@ def test_swiglu_gate_first():
     torch.testing.assert_close(plain.swiglu(x, w, "p."), want, atol=1e-5, rtol=1e-5)
 
 
-def test_norm_sits_before_rotation_and_values_are_not_normed(folder_b):
-    """QK-norm before RoPE, V untouched (rollout/monkey_patch/qwen3.py:29-31): scaling q_norm's weight
-    scales the scores; scaling v_proj scales the attention output linearly."""
+def test_values_are_not_normed_and_the_norm_removes_the_scale_of_q(folder_b):
+    """V is untouched (rollout/monkey_patch/qwen3.py:31): scaling v_proj scales the attention output
+    linearly; q passes a per-head norm (qwen3.py:29): scaling q_proj changes nothing."""
     cfg, w = plain.read_folder(folder_b)
     x = torch.randn(7, cfg["hidden_size"])
     pos = torch.arange(7)
@@ -118,6 +118,55 @@ def test_norm_sits_before_rotation_and_values_are_not_normed(folder_b):
     w3["model.layers.0.self_attn.q_proj.weight"] = 5 * w["model.layers.0.self_attn.q_proj.weight"]
     torch.testing.assert_close(plain.attention_part(x, w3, "model.layers.0.self_attn.", cfg, pos), base,
                                atol=1e-4, rtol=1e-3)      # the per-head norm removes the scale of q
+
+
+def test_norm_sits_before_rotation(folder_b):
+    """QK-norm first, rotation after it (rollout/monkey_patch/qwen3.py:29-30 norm q and k; the
+    rotation happens later, inside the attention kernel, rollout/attention.py:89-96, 116-125). With a
+    constant norm weight the two orders give the same vectors (a rotation keeps a head's mean square),
+    so the weights here differ strongly along the head: then w * rotate(x) and rotate(w * x) differ,
+    because the rotation mixes element j with element j + D/2, which carry different weights.
+    The scores are written out here for one head from the norm, the angles and the rotation alone."""
+    cfg, w = plain.read_folder(folder_b)
+    pre = "model.layers.0.self_attn."
+    D, eps, theta = cfg["head_dim"], cfg["rms_norm_eps"], cfg["rope_theta"]
+    w = dict(w)
+    w[pre + "q_norm.weight"] = torch.linspace(0.2, 3.0, D)
+    w[pre + "k_norm.weight"] = torch.linspace(2.5, 0.3, D) ** 2
+    T = 9
+    x = torch.randn(T, cfg["hidden_size"])
+    pos = torch.arange(40, 40 + T)                        # far from 0, so that the angles are large
+    got = plain.attention_part(x, w, pre, cfg, pos)
+
+    def by_hand(norm_first):
+        q = (x @ w[pre + "q_proj.weight"].T).view(T, -1, D)
+        k = (x @ w[pre + "k_proj.weight"].T).view(T, -1, D)
+        v = (x @ w[pre + "v_proj.weight"].T).view(T, -1, D)
+        inv = 1.0 / theta ** (torch.arange(0, D // 2).float() / (D // 2))
+        ang = pos.float()[:, None] * inv[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+        def norm(t, weight):
+            return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps) * weight
+
+        def rotate(t):
+            a, b = t[..., :D // 2], t[..., D // 2:]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+        if norm_first:
+            q, k = rotate(norm(q, w[pre + "q_norm.weight"])), rotate(norm(k, w[pre + "k_norm.weight"]))
+        else:
+            q, k = norm(rotate(q), w[pre + "q_norm.weight"]), norm(rotate(k), w[pre + "k_norm.weight"])
+        out = torch.zeros(T, q.shape[1], D)
+        G = q.shape[1] // k.shape[1]
+        for h in range(q.shape[1]):
+            s = (q[:, h] @ k[:, h // G].T) * D ** -0.5
+            s = s.masked_fill(torch.ones(T, T, dtype=torch.bool).triu(1), float("-inf"))
+            out[:, h] = s.softmax(-1) @ v[:, h // G]
+        return out.reshape(T, -1) @ w[pre + "o_proj.weight"].T
+
+    torch.testing.assert_close(got, by_hand(True), atol=1e-5, rtol=1e-4)
+    wrong = by_hand(False)
+    assert (got - wrong).abs().max() > 50 * (got - by_hand(True)).abs().max() + 1e-3   # the other order is another function
 
 
 def test_whole_model_shapes_and_tying(folder_a, folder_b):
