@@ -132,6 +132,75 @@ def decode_steps(runner, ids, steps, warmup, vocab):
     return time.perf_counter() - t0
 
 
+def measured_peaks(runner, dtype):
+    """What this machine reaches, measured in this run: GB/s of a plain read-only kernel over 2 GiB that
+    nothing else touches, and TFLOP/s of one library product of the prefill's largest shape
+    (2,048 x 4,096 times 12,288 x 4,096, random operands, the compute dtype)."""
+    import torch
+    ops = runner.rt.ops
+    out = {}
+    buf = torch.empty(2 << 30, dtype=torch.uint8, device="cuda:0")
+    buf.random_(0, 256)
+    best = None
+    for _ in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ops.stream_read(buf)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    out["read_GBs"] = round(buf.numel() / best / 1e9, 1)
+    del buf
+    td = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    a = torch.randn(2048, 4096, device="cuda:0").to(td)
+    b = torch.randn(12288, 4096, device="cuda:0").to(td)
+    reps, best = 8, None
+    for _ in range(4):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            torch.matmul(a, b.t())
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / reps
+        best = dt if best is None else min(best, dt)
+    out["product_TFLOPs"] = round(2.0 * 2048 * 4096 * 12288 / best / 1e12, 1)
+    torch.cuda.empty_cache()
+    return out
+
+
+def kernel_split(run, steps):
+    """Device time of `steps` calls of run() by kernel, from a profiler pass of its own (outside every
+    timed region; what rollout/utils/prof_graph.py:64-101 does for the reference's decode): the ten
+    kernels that take the most time, in microseconds per call, the rest as "other", and the sum."""
+    import re
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+    try:
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            for _ in range(steps):
+                run()
+            torch.cuda.synchronize()
+        per = {}
+        for e in prof.key_averages():
+            us = getattr(e, "self_device_time_total", 0) or getattr(e, "self_cuda_time_total", 0)
+            if us > 0 and not e.key.startswith("Memcpy") and not e.key.startswith("Memset"):
+                name = re.sub(r"<.*", "", re.sub(r"^void ", "", e.key))
+                name = name if len(name) <= 48 else name[:45] + "..."
+                calls, total = per.get(name, (0, 0.0))
+                per[name] = (calls + e.count, total + us)
+        if not per:
+            return {"error": "the profiler saw no kernels"}
+        top = sorted(per.items(), key=lambda kv: -kv[1][1])
+        out = {name: {"us": round(us / steps, 1), "calls": round(calls / steps, 1)} for name, (calls, us) in top[:10]}
+        rest = sum(us for _, (_, us) in top[10:])
+        if rest > 0:
+            out["other"] = {"us": round(rest / steps, 1), "calls": round(sum(c for _, (c, _) in top[10:]) / steps, 1)}
+        out["sum_us"] = round(sum(us for _, us in per.values()) / steps, 1)
+        return out
+    except Exception as error:          # a measurement beside the bench: its failure is reported, not raised
+        return {"error": f"{type(error).__name__}: {error}"[:200]}
+
+
 def release(runner, ids):
     for rid in ids:
         runner.free_request(rid)
@@ -281,40 +350,68 @@ def main():
                                use_graphs=not args.no_graphs, tune_products=not args.no_tune)
     V = cfg.vocab_size
 
+    def roofline(batch, ms, new_before, steps):
+        """Bytes a decode step has to read (every weight once, the cache of the live requests at their
+        mean length over the timed steps) over its time, against the published and the measured read rate."""
+        mean_ctx = CONTEXT + new_before + (steps + 1) / 2.0
+        step_bytes = weight_bytes(cfg, elt) + batch * mean_ctx * kv_bytes_per_token(cfg, elt)
+        got = step_bytes / (ms * 1e-3) / 1e9
+        r = {"bound": "hbm", "achieved": round(got, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+             "frac": round(got / PEAK_HBM_GBS, 4)}
+        if peaks:
+            r["measured_peak"] = peaks["read_GBs"]
+            r["frac_of_measured"] = round(got / peaks["read_GBs"], 4)
+        return r
+
+    peaks = None if args.no_points else measured_peaks(runner, args.dtype)
+
     # ---- headline: decode at the given batch
     ids = seat_requests(runner, args.batch, CONTEXT)
     secs = decode_steps(runner, ids, args.steps, args.warmup, V)
-    release(runner, ids)
     ms_step = secs / args.steps * 1e3
     value = args.batch * args.steps / secs
-    mean_ctx = CONTEXT + args.warmup + (args.steps + 1) / 2.0
-    step_bytes = weight_bytes(cfg, elt) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elt)
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    headline = roofline(args.batch, ms_step, args.warmup, args.steps)
+    kernels = None
+    if not args.no_points:              # where the step's time goes, from a pass of its own after the timed one
+        def one_step():
+            n = args.batch
+            t = runner.decode_launch(ids, None, [0.0] * n, [0] * n, [1.0] * n, [0.0] * n, feed_rows=list(range(n)))
+            runner.decode_collect(t)
+        kernels = kernel_split(one_step, 4)
+    release(runner, ids)
 
-    points, prefill = {}, None
+    points, point_rooflines, prefill, prefill_kernels = {}, {}, None, None
     if not args.no_points:
         for b in (1, 64):
             ids = seat_requests(runner, b, CONTEXT)
             k = max(8, min(args.steps, 32))
-            s = decode_steps(runner, ids, k, min(args.warmup, 4), V)
+            w = min(args.warmup, 4)
+            s = decode_steps(runner, ids, k, w, V)
             release(runner, ids)
             points[f"decode_b{b}"] = round(b * k / s, 1)
+            point_rooflines[f"decode_b{b}"] = dict(roofline(b, s / k * 1e3, w, k), ms_per_step=round(s / k * 1e3, 4))
         # ---- prefill of one 2,048-token prompt, logits at the last place
         from return_amd.engine import StepEntry
         prompt = [(13 * i + 5) % V for i in range(PREFILL_TOKENS)]
         times = []
-        for it in range(4):
+
+        def one_prefill():
             runner.add_request("p")
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
             out = runner.step([StepEntry("p", prompt, [PREFILL_TOKENS - 1])])
             out.sum().item()
-            times.append(time.perf_counter() - t0)
             runner.free_request("p")
+        for it in range(4):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            one_prefill()
+            times.append(time.perf_counter() - t0)
         pf = min(times[1:])
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
         prefill = {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS,
-                   "ms": round(pf * 1e3, 3),
-                   "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pf / PEAK_FLOPS[args.dtype], 4)}
+                   "ms": round(pf * 1e3, 3), "frac": round(flops / pf / PEAK_FLOPS[args.dtype], 4),
+                   "measured_peak_TFLOPs": peaks["product_TFLOPs"],
+                   "frac_of_measured": round(flops / pf / (peaks["product_TFLOPs"] * 1e12), 4)}
+        prefill_kernels = kernel_split(one_prefill, 2)
 
     line = {
         "metric": "decode tok/s (Qwen3-8B shape, random weights)",
@@ -330,9 +427,14 @@ def main():
                    "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
                    "hip_graphs": not args.no_graphs, "tuned_products": not args.no_tune,
                    "weights": "random N(0,0.02)"},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "roofline": headline,
     }
+    if peaks:
+        line["measured"] = peaks
+    if kernels:
+        line["kernels"] = kernels
+    if prefill_kernels:
+        line["prefill_kernels"] = prefill_kernels
     plan = getattr(runner.rt.ops, "product_plan", None)
     if plan:            # where the measurement at load replaced the rule: rows x N x K -> way
         line["product_plan"] = {f"{rows}x{n}x{k}{'g' if gated else ''}": how
@@ -342,6 +444,7 @@ def main():
     if points:
         points[f"decode_b{args.batch}"] = round(value, 1)
         line["points"] = points
+        line["point_rooflines"] = point_rooflines
     print(json.dumps(line))
     return 0
 

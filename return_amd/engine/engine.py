@@ -62,6 +62,10 @@ class Engine:
         self.decode_seconds = 0.0
         self.prefill_seconds = 0.0
         self.steps = 0
+        self._t_start = time.perf_counter()
+        self._decode_streak = 0             # steps that only decoded since the last step with a prompt portion
+        self._streak_total = 0
+        self._streak_count = 0
 
     # ------------------------------------------------------------------ requests
     def submit(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
@@ -117,6 +121,7 @@ class Engine:
         return self.runner.step_launch(entries, *options, feed=feed)
 
     def _book(self, plan, sampled, t0):
+        only_decode = all(len(e.tokens) == 1 and e.request.output for e in plan.entries if not e.request.finished)
         for e in plan.entries:
             if e.request.finished:
                 continue
@@ -127,10 +132,15 @@ class Engine:
         ended = self.scheduler.finish_step(plan, sampled)
         dt = time.perf_counter() - t0
         self.step_seconds += dt
-        if all(len(e.tokens) == 1 and e.sample for e in plan.entries):
+        if only_decode:
             self.decode_seconds += dt               # steps that only decode
+            self._decode_streak += 1
         else:
             self.prefill_seconds += dt              # steps that bring prompt portions (decoded tokens beside them)
+            if self._decode_streak > 0:             # a run of decode steps ends (rollout/engine.py:361-364)
+                self._streak_total += self._decode_streak
+                self._streak_count += 1
+                self._decode_streak = 0
         self.steps += 1
         return ended
 
@@ -217,12 +227,20 @@ class Engine:
 
     def stats(self) -> dict:
         cache = self.runner.cache
+        run = time.perf_counter() - self._t_start
         return {"steps": self.steps, "prefill_tokens": self.prefill_tokens,
                 "decode_tokens": self.decode_tokens, "step_seconds": self.step_seconds,
                 # the reference's decode_tps / prefill_tps (rollout/engine.py:104-110): tokens over the
                 # time of the steps of that kind (decoded tokens of mixed steps count as decoded)
                 "decode_tps": self.decode_tokens / self.decode_seconds if self.decode_seconds > 0 else None,
                 "prefill_tps": self.prefill_tokens / self.prefill_seconds if self.prefill_seconds > 0 else None,
+                # share of the time since the engine was made that went into steps of each kind, and the
+                # mean number of decode-only steps between two steps that brought prompt portions
+                # (decode_duty, prefill_duty, decode_streak of rollout/engine.py:113-125)
+                "run_seconds": run,
+                "decode_duty": self.decode_seconds / run if run > 0 else 0.0,
+                "prefill_duty": self.prefill_seconds / run if run > 0 else 0.0,
+                "decode_streak": self._streak_total / self._streak_count if self._streak_count else None,
                 "running": len(self.scheduler.running), "waiting": len(self.scheduler.waiting),
                 "resident": len(self.scheduler.resident),
                 "kv_used": [g.pages.in_use() for g in cache.groups],

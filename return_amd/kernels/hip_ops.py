@@ -74,6 +74,7 @@ def _declare(lib):
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "ra_attention_prefill_tile_rows": [I],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
+        "ra_stream_read": [P, L, P, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -672,6 +673,19 @@ class HipOps:
         ends = [s + min(off + rows, q) for q, s in zip(step.q_lens, step.q_starts) if q != 1
                 for off in range(0, q, rows)]
         return 2 if max(ends) * len(ends) >= 1.4 * sum(ends) else 1
+
+    # ------------------------------------------------------------------ measurement
+    def stream_read(self, t, workgroups=0):
+        """Reads every byte of tensor t once with a plain read-only kernel (one workgroup per CU unless
+        given); returns the words it folded them into. For measuring the machine's read rate."""
+        self._want(t, "tensor to read")
+        n = t.numel() * t.element_size()
+        if n == 0 or n % 16 or t.data_ptr() % 16:
+            raise KernelError(f"stream_read: {n} bytes at {t.data_ptr():#x} are no whole 16-byte pieces")
+        g = int(workgroups) or self.cu_count
+        out = torch.empty(g, dtype=torch.int32, device=self.device)
+        self._check(self.lib.ra_stream_read(_ptr(t), n, _ptr(out), g, self._stream()), "stream_read")
+        return out
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, top_p, u):

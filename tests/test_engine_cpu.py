@@ -350,3 +350,24 @@ def test_a_step_that_cannot_start_fails_its_requests_and_frees_them(folder_a, mo
     out = eng.generate([[7, 8, 9]], sp)[0]                 # the step that was under way is collected, then life goes on
     assert out.num_tokens == 5 and not eng.runner.cache.live
     eng.runner.cache.check_invariants()
+
+
+def test_duty_and_decode_streak(folder_a):
+    """The reference's counters (rollout/engine.py:84-125, 361-364, 403): the share of the run that went
+    into steps of each kind, and the mean run of decode-only steps between steps that brought prompts."""
+    V = TINY_A["vocab_size"]
+    eng = engine_for(folder_a, max_reside=2, max_token=512, lookahead=False)
+    assert eng.stats()["decode_streak"] is None and eng.stats()["decode_duty"] == 0.0
+    sp = SamplingParams(temperature=0.0, max_new_tokens=5)
+    # two at once: one prompt step, then four steps that only decode; then the same again
+    for turn in range(2):
+        eng.generate([tt.random_tokens(V, 9, seed=turn), tt.random_tokens(V, 20, seed=7 + turn)], sp)
+    st = eng.stats()
+    assert st["steps"] == 10 and eng._decode_streak == 4        # the run under way is not counted yet
+    assert st["decode_streak"] == 4.0                           # one closed run of four
+    eng.generate([tt.random_tokens(V, 3, seed=5)], SamplingParams(temperature=0.0, max_new_tokens=2))
+    st = eng.stats()
+    assert st["decode_streak"] == 4.0 and eng._decode_streak == 1
+    assert 0 < st["decode_duty"] < 1 and 0 < st["prefill_duty"] < 1
+    assert st["decode_duty"] + st["prefill_duty"] <= 1.0 + 1e-9
+    assert abs(st["decode_duty"] * st["run_seconds"] - eng.decode_seconds) < 1e-6
