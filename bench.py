@@ -184,7 +184,10 @@ def kernel_split(run, steps):
         for e in prof.key_averages():
             us = getattr(e, "self_device_time_total", 0) or getattr(e, "self_cuda_time_total", 0)
             if us > 0 and not e.key.startswith("Memcpy") and not e.key.startswith("Memset"):
-                name = re.sub(r"<.*", "", re.sub(r"^void ", "", e.key))
+                name = re.sub(r"[<(].*", "", re.sub(r"^void ", "", e.key))
+                tile = re.search(r"_(MT\d+x\d+x\d+)_", e.key)
+                if e.key.startswith(("Cijk_", "Custom_Cijk_")) and tile:     # the library's products differ by their tile
+                    name = "library product " + tile.group(1)
                 name = name if len(name) <= 48 else name[:45] + "..."
                 calls, total = per.get(name, (0, 0.0))
                 per[name] = (calls + e.count, total + us)

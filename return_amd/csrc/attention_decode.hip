@@ -220,16 +220,19 @@ void attn_decode_kernel(
     const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int h0 = kvh * group + hb * DEC_MAX_GROUP;             // first query head of this wave
     const int G = min(DEC_MAX_GROUP, group - hb * DEC_MAX_GROUP);  // and how many it has
-    const int t = cu_q[seg];
+    // (the request's four numbers are asked for together; cu_q == nullptr: every request brings one
+    // token, so its row is its number, and the loads of q need not wait for a table)
+    const int t = cu_q ? cu_q[seg] : seg;
     const int pos_q = q_start[seg];
     const int start = kv_start[seg];
+    const int first_page = cu_pages[seg];
     // A merging workgroup cuts its own request into merge_waves even splits (counted from
     // position 0), whatever the longest request of the step is.
     if (merge_waves > 1) split_tokens = max(1, (pos_q + DEC_CHUNK * merge_waves) / (DEC_CHUNK * merge_waves)) * DEC_CHUNK;
     const DecodeRange rg = decode_range(pos_q, start, window, split_tokens, sp);
     const bool empty = rg.lo > rg.hi;            // a split beyond the request's keys
     if (empty && merge_waves == 1) return;       // (in a merging workgroup the wave stays for the barrier, with no keys)
-    const int* pt = page_table + cu_pages[seg];
+    const int* pt = page_table + first_page;
     const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
 
     // query operand: lane (n, g) holds head h0+n, d = 32j + 8g .. +7 (and D-16+8g.. for the tail)
@@ -554,38 +557,60 @@ extern "C" int ra_dec_part_2(DEC_PART_ARGS);
 extern "C" int ra_dec_part_3(DEC_PART_ARGS);
 
 // Merge of the splits, in split order: out = sum_s acc_s * w_s / sum_s l_s * w_s, w_s = exp(m_s - m).
+// The kernel is a chain of loads that wait for each other (the request's tables, then the splits'
+// maxima, then their sums), and each link costs about a microsecond after a kernel that wrote them.
+// So the first COMBINE_AHEAD splits' maxima and sums are asked for at once with the tables, before it
+// is known how many splits hold keys: what a split beyond them left in memory is read and not used.
+// Every thread forms the weights itself (the same numbers in the same order), so that no thread waits
+// for another.
+#define COMBINE_AHEAD 16
 __global__ __launch_bounds__(128) void attn_decode_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
     const int* __restrict__ kv_start, const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ seg_ids, int Hq, int D, int window, int split_tokens, int max_splits) {
-    extern __shared__ float w_s[];                     // [ns]
-    __shared__ float stat[2];
     const int di = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
-    const int seg = seg_ids ? seg_ids[di] : di;
-    const int t = cu_q[seg];
-    const DecodeRange rg = decode_range(q_start[seg], kv_start[seg], window, split_tokens, 0);
-    const int ns = min(rg.n_splits, max_splits);
     const float* pm = part_ml + ((size_t)di * Hq + head) * max_splits * 2;
     const float* pa = part_acc + ((size_t)di * Hq + head) * max_splits * D;
-    if (tid < 64) {                                    // first wave: maximum, weights, sum in split order
-        float m = -INFINITY;                           // (the maxima are base-2 exponents)
-        for (int s = tid; s < ns; s += 64) m = fmaxf(m, pm[2 * s]);
-        m = wave_max(m);
-        for (int s = tid; s < ns; s += 64) w_s[s] = __builtin_amdgcn_exp2f(pm[2 * s] - m);
-        if (tid == 0) {
-            float l = 0.f;
-            for (int s = 0; s < ns; ++s) l += pm[2 * s + 1] * __builtin_amdgcn_exp2f(pm[2 * s] - m);
-            stat[0] = l > 0.f ? 1.0f / l : 0.f;
+    const int d0 = min(tid, D - 1), d1 = min(tid + 128, D - 1);       // this thread's columns (D <= 256), clamped for the loads
+    float2_t ml[COMBINE_AHEAD];
+    float a0[COMBINE_AHEAD], a1[COMBINE_AHEAD];
+#pragma unroll
+    for (int s = 0; s < COMBINE_AHEAD; ++s) {
+        const int sc = min(s, max_splits - 1);
+        ml[s] = *reinterpret_cast<const float2_t*>(pm + 2 * sc);
+        a0[s] = pa[(size_t)sc * D + d0];
+        a1[s] = pa[(size_t)sc * D + d1];
+    }
+    const int seg = seg_ids ? seg_ids[di] : di;
+    const int t = cu_q ? cu_q[seg] : seg;
+    const DecodeRange rg = decode_range(q_start[seg], kv_start[seg], window, split_tokens, 0);
+    const int ns = min(rg.n_splits, max_splits);
+    float m = -INFINITY;                                   // (the maxima are base-2 exponents)
+#pragma unroll
+    for (int s = 0; s < COMBINE_AHEAD; ++s) m = s < ns ? fmaxf(m, ml[s][0]) : m;
+#pragma unroll 8
+    for (int s = COMBINE_AHEAD; s < ns; ++s) m = fmaxf(m, pm[2 * s]);
+    float l = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (int s = 0; s < COMBINE_AHEAD; ++s) {
+        if (s < ns) {
+            const float w = __builtin_amdgcn_exp2f(ml[s][0] - m);
+            l += ml[s][1] * w;
+            o0 = fmaf(a0[s], w, o0);
+            o1 = fmaf(a1[s], w, o1);
         }
     }
-    __syncthreads();
-    const float inv = stat[0];
-    for (int d = tid; d < D; d += 128) {
-        float o = 0.f;
 #pragma unroll 8
-        for (int s = 0; s < ns; ++s) o = fmaf(pa[(size_t)s * D + d], w_s[s], o);
-        out[((size_t)t * Hq + head) * D + d] = from_f<bf16>(o * inv);
+    for (int s = COMBINE_AHEAD; s < ns; ++s) {
+        const float w = __builtin_amdgcn_exp2f(pm[2 * s] - m);
+        l += pm[2 * s + 1] * w;
+        o0 = fmaf(pa[(size_t)s * D + d0], w, o0);
+        o1 = fmaf(pa[(size_t)s * D + d1], w, o1);
     }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16* o = out + ((size_t)t * Hq + head) * D;
+    if (tid < D) o[tid] = from_f<bf16>(o0 * inv);
+    if (tid + 128 < D) o[tid + 128] = from_f<bf16>(o1 * inv);
 }
 
 // part_acc: fp32 [n_dec, Hq, max_splits, D]; part_ml: fp32 [n_dec, Hq, max_splits, 2].
@@ -633,8 +658,7 @@ static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const 
     if (rc != RA_OK) return rc;
     if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
     if (merge) return RA_OK;
-    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128),
-                       (size_t)max_splits * sizeof(float), st, pa, pm, (bf16*)out, kv_start, cu_q,
+    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128), 0, st, pa, pm, (bf16*)out, kv_start, cu_q,
                        q_start, seg_ids, Hq, D, window, split_tokens, max_splits);
     return ra_launch_status();
 }
@@ -655,7 +679,8 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
 // The same for requests whose new token has not been prepared: qkv [tokens, (Hq + 2 Hkv) D] as the
 // projection left it. The kernel norms (w_q, w_k [D]; nullptr: no norm) and rotates (cos, sin
 // [positions, D/2] at the request's position; nullptr: no rotation) q and k itself and writes k and
-// v of the new token into the pools. Head sizes 64, 128, 192, 256.
+// v of the new token into the pools. Head sizes 64, 128, 192, 256. cu_q == nullptr: every request brings
+// exactly one token and row i of qkv and of out is request i (no seg_ids then).
 extern "C" int ra_attention_decode_fused_bf16(const void* qkv, void* out, void* part_acc, void* part_ml,
                                               void* k_pool, void* v_pool, const int* page_table,
                                               const int* cu_pages, const int* kv_start, const int* cu_q,
@@ -665,7 +690,7 @@ extern "C" int ra_attention_decode_fused_bf16(const void* qkv, void* out, void* 
                                               const float* w_k, float eps, const float* cos_t,
                                               const float* sin_t, int merge, void* stream) {
     if (qkv == nullptr || D % 64 != 0 || (w_q == nullptr) != (w_k == nullptr) ||
-        (cos_t == nullptr) != (sin_t == nullptr))
+        (cos_t == nullptr) != (sin_t == nullptr) || (cu_q == nullptr && seg_ids != nullptr))
         return RA_ERR_ARG;
     DecodeFused fz = {(const bf16*)qkv, w_q, w_k, eps, cos_t, sin_t, (bf16*)k_pool, (bf16*)v_pool};
     return decode_launch(nullptr, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,

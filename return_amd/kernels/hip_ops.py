@@ -655,8 +655,9 @@ class HipOps:
             part_ml = torch.empty(nd, n_q, max_splits, 2, dtype=torch.float32, device=self.device)
         self._check(self.lib.ra_attention_decode_fused_bf16(
             _ptr(qkv), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(k_pool), _ptr(v_pool),
-            _ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start),
-            _ptr(step.decode_segs), nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
+            # (no cu_q: every request brings one token, checked above, so request i is row i)
+            _ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), None, _ptr(step.q_start),
+            None, nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
             _ptr(w_q), _ptr(w_k), float(eps), _ptr(cos) if R else None, _ptr(sin) if R else None,
             1 if merge else 0, self._stream()), "attention_decode_fused_bf16")
         return True
