@@ -320,9 +320,78 @@ def long_32b(args):
             "prefill": pre(ctx, t1 - t0, n), "prefill_long": pre(long_ctx, best, 1)}
 
 
+def contexts_8b(args):
+    """The 8B shape at further context lengths: decode at batch 1, 8 and 64 over contexts of 8,192 and
+    32,768 tokens (batch 64 at 32,768 would need 309 GB of cache and is left out), each with the
+    fraction of the read roofline, a prefill of 16,384 tokens in one portion, and what sampling with
+    top_p = 0.9 costs at 64 rows of this vocabulary beside greedy sampling. value: decode tok/s at
+    batch 8 over 8,192 tokens."""
+    import torch
+    from return_amd.engine import StepEntry
+    elt = 2 if args.dtype == "bfloat16" else 4
+    points = {}
+    cfg = runner = None
+    for ctx, batches in ((8192, (1, 8, 64)), (32768, (1, 8))):
+        del runner
+        torch.cuda.empty_cache()
+        cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(batches), use_graphs=not args.no_graphs,
+                                   tune_products=not args.no_tune, max_token=max(batches) * (ctx + 256))
+        for b in batches:
+            ids = seat_requests(runner, b, ctx)
+            k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+            secs = decode_steps(runner, ids, k, w, cfg.vocab_size)
+            release(runner, ids)
+            ms = secs / k * 1e3
+            step_bytes = weight_bytes(cfg, elt) + b * (ctx + w + (k + 1) / 2.0) * kv_bytes_per_token(cfg, elt)
+            got = step_bytes / (ms * 1e-3) / 1e9
+            points[f"decode_b{b}_ctx{ctx}"] = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4),
+                                              "GBs": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4)}
+    # ---- sampling at 64 rows of the full vocabulary: greedy against temperature 1 with top_p 0.9
+    logits = torch.randn(64, cfg.vocab_size, device="cuda:0") * 3.0
+    sampling = {}
+    for name, temp, top_p in (("greedy", 0.0, 1.0), ("top_p_0.9", 1.0, 0.9), ("top_k_50", 1.0, 1.0)):
+        best = None
+        for _ in range(5):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.sample(logits, [temp] * 64, [50 if name == "top_k_50" else 0] * 64, [top_p] * 64, [0.37] * 64)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        sampling[name + "_us"] = round(best * 1e6, 1)
+    del logits
+    # ---- one prompt of 16,384 tokens in one portion
+    n = 16384
+    del runner
+    torch.cuda.empty_cache()
+    cfg, runner = build_runner(args.layers, args.dtype, max_reside=2, use_graphs=False, tune_products=False,
+                               max_token=n + 256, max_step_tokens=n, prefill_chunk=n)
+    prompt = [(13 * i + 5) % cfg.vocab_size for i in range(n)]
+    times = []
+    for _ in range(3):
+        runner.add_request("p")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry("p", prompt, [n - 1])]).sum().item()
+        times.append(time.perf_counter() - t0)
+        runner.free_request("p")
+    pf = min(times[1:])
+    head = points["decode_b8_ctx8192"]
+    return {"metric": "decode tok/s at batch 8 over 8,192-token contexts (Qwen3-8B shape, random weights)",
+            "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": max(8, min(args.steps, 32)),
+            "warmup": min(args.warmup, 4), "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic",
+            "config": shape_of(cfg, model="Qwen3-8B shape", global_batch=8, seq_len=8192, hip_graphs=not args.no_graphs,
+                               weights="random N(0,0.02)"),
+            "points": points, "sampling_64_rows": sampling,
+            "prefill_16384": {"value": round(n / pf, 1), "tokens": n, "ms": round(pf * 1e3, 2),
+                              "frac": round(prefill_flops(cfg, n) / pf / PEAK_FLOPS[args.dtype], 4)}}
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="decode_8b", choices=["decode_8b", "continuous_4b", "long_32b"],
+    ap.add_argument("--workload", default="decode_8b",
+                    choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -346,7 +415,8 @@ def main():
         print("bench.py: no GPU visible")
         return 1
     if args.workload != "decode_8b":
-        print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b}[args.workload](args)))
+        print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
+                          "contexts_8b": contexts_8b}[args.workload](args)))
         return 0
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),

@@ -668,6 +668,34 @@ def test_sample_matches_plain_draw(ops, ref, V):
                                atol=1e-4, rtol=1e-5)
 
 
+def test_sample_at_the_full_vocabulary(ops):
+    """top-k and top-p at a vocabulary of 151,936 (the threshold search over seven passes and its
+    bins): every row's token is where the plain distribution's running sum, in vocabulary order,
+    passes the row's uniform number; peaked and flat rows, ties above the boundary (tokens that tie
+    with the boundary value itself are all kept here, one by one in the plain rule), k = 1, p near 0."""
+    from tests.plain import qwen3_plain as plain
+    V, M = 151936, 32
+    logits = rnd(M, V, seed=73, scale=3.0)
+    logits[1] = (logits[1] * 0.05)                                # flat: top-p keeps tens of thousands
+    logits[2, 1000:1040] = logits[2].max() + 1.0                  # forty tokens tie at the top
+    logits[3, 5000:5003] = logits[3].max()                        # three more tokens tie with the largest (all above the boundary)
+    g = torch.Generator().manual_seed(11)
+    u = torch.rand(M, generator=g).to(DEV)
+    temp = torch.tensor([0.7, 1.0, 1.3, 0.9] * (M // 4), device=DEV)
+    top_k = torch.tensor([0, 0, 50, 0, 20, 1, 0, 3000] * (M // 8), dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([0.9, 0.95, 1.0, 0.5, 0.8, 1.0, 0.01, 0.99] * (M // 8), device=DEV)
+    out = ops.sample(logits, temp, top_k, top_p, u).cpu()
+    for r in range(M):
+        d = plain.sample_distribution(logits[r].cpu(), float(temp[r]), int(top_k[r]), float(top_p[r]))
+        tok = int(out[r, 0])
+        assert d[tok] > 0, f"row {r}: token {tok} is not among the kept ones"
+        c = d.cumsum(0)
+        before = float(c[tok - 1]) if tok else 0.0
+        assert before - 1e-4 <= float(u[r]) <= float(c[tok]) + 1e-4, (r, tok, before, float(u[r]), float(c[tok]))
+        lp = out[r, 1:2].contiguous().view(torch.float32)
+        assert abs(float(lp) - plain.chosen_logprob(logits[r].cpu(), tok)) < 1e-3
+
+
 def test_sample_distribution(ops):
     """Plain temperature sampling draws from softmax(logits / T): chi-square on a tiny vocabulary."""
     V, N = 7, 20000
