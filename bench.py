@@ -184,7 +184,9 @@ def kernel_split(run, steps):
         for e in prof.key_averages():
             us = getattr(e, "self_device_time_total", 0) or getattr(e, "self_cuda_time_total", 0)
             if us > 0 and not e.key.startswith("Memcpy") and not e.key.startswith("Memset"):
-                name = re.sub(r"[<(].*", "", re.sub(r"^void ", "", e.key))
+                name = re.sub(r"^void ", "", e.key)
+                # (the hand-written products keep their template arguments: they say which form ran)
+                name = re.sub(r"\(.*", "", name) if name.startswith("gemm_") else re.sub(r"[<(].*", "", name)
                 tile = re.search(r"_(MT\d+x\d+x\d+)_", e.key)
                 if e.key.startswith(("Cijk_", "Custom_Cijk_")) and tile:     # the library's products differ by their tile
                     name = "library product " + tile.group(1)
@@ -402,6 +404,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel from the host instead of replaying HIP graphs")
+    ap.add_argument("--no-defer-norms", action="store_true",
+                    help="run every RMSNorm as a kernel of its own instead of inside the products around it")
     ap.add_argument("--no-tune", action="store_true",
                     help="choose the kernel of every projection by rule instead of measuring at load "
                          "(keeps the measuring launches out of a profile)")
@@ -420,7 +424,8 @@ def main():
         return 0
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),
-                               use_graphs=not args.no_graphs, tune_products=not args.no_tune)
+                               use_graphs=not args.no_graphs, tune_products=not args.no_tune,
+                               defer_norms=not args.no_defer_norms)
     V = cfg.vocab_size
 
     def roofline(batch, ms, new_before, steps):
@@ -499,7 +504,7 @@ def main():
                    "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": PAGE,
                    "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
                    "hip_graphs": not args.no_graphs, "tuned_products": not args.no_tune,
-                   "weights": "random N(0,0.02)"},
+                   "norms_in_products": not args.no_defer_norms, "weights": "random N(0,0.02)"},
         "roofline": headline,
     }
     if peaks:

@@ -59,7 +59,7 @@ def cmd_generate(args) -> int:
     engine = Engine(args.model, max_token=args.max_token, max_reside=args.max_reside, dtype=args.dtype,
                     page_size=args.page_size, seed=args.seed, max_step_tokens=args.max_step_tokens,
                     prefill_chunk=args.prefill_chunk, use_graphs=not args.no_graphs,
-                    tune_products=not args.no_tune)
+                    tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
     # Requests are run together until a session_id comes again: that request is a later turn of the
     # session (the reference keeps a session's cache for its next request, rollout/engine.py:286-306,
     # which sends the whole conversation again, 266-274). A session's cache is kept while more of
@@ -120,6 +120,8 @@ def main(argv=None) -> int:
     g.add_argument("--seed", type=int, default=0)
     g.add_argument("--no-graphs", action="store_true",
                    help="launch every kernel of a decode step from the host instead of replaying HIP graphs")
+    g.add_argument("--no-defer-norms", action="store_true",
+                   help="run every RMSNorm as a kernel of its own instead of inside the products around it")
     g.add_argument("--no-tune", action="store_true",
                    help="choose the kernel of every projection by rule instead of measuring at load")
     g.add_argument("--requests", help="file of JSON lines (or - for standard input), one request each")

@@ -21,6 +21,7 @@ class EngineConfig:
     use_graphs: bool = True            # replay decode-only steps from captured HIP graphs (USE_CUDA_GRAPH of the reference)
     lookahead: bool = True             # launch every step before the sampled tokens of the one before it are read
     tune_products: bool = True         # measure at load which kernel forms each projection fastest at few rows
+    defer_norms: bool = True           # steps of few rows: finish every RMSNorm inside the products around it (two kernels less per layer)
     seed: int = 0                      # base seed of the sampling streams
     device: str = "cuda:0"
 

@@ -50,6 +50,8 @@ class ModelRunner:
         _, build_spec = lookup_architecture(config.architecture)
         self.spec = build_spec(config)
         self.rt = Runtime(ec.device, ec.dtype, ops=ops)
+        if hasattr(self.rt.ops, "defer_norms"):
+            self.rt.ops.defer_norms = bool(ec.defer_norms)
         if weights is None:
             if model_dir is None:
                 raise ValueError("ModelRunner got a configuration but no weights")

@@ -12,6 +12,7 @@ from typing import Optional
 
 import torch
 
+from ..parts.runtime import ScaledRows
 from . import build as _build
 
 _F32, _BF16 = 0, 1
@@ -66,6 +67,8 @@ def _declare(lib):
         "ra_gemm_resident_fits": [I, I, I],
         "ra_gemm_sweep_bf16": [P, P, P, I, I, I, I, I, I, P],
         "ra_gemm_sweep_fits": [I, I],
+        "ra_gemm_sweep_workgroups": [I, I],
+        "ra_gemm_sweep_norm_bf16": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, I, P],
@@ -111,6 +114,7 @@ class HipOps:
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
         self.own_gemm = False                # True: bf16 products of many rows use the hand-written MFMA kernel
+        self.defer_norms = True              # finish RMSNorms inside the products around them where the sweep takes both
         try:                                 # whether the library multiplies bf16 operands into fp32 results
             a = torch.ones(1, 8, dtype=torch.bfloat16, device=self.device)
             self._library_fp32_out = torch.mm(a, a.t(), out_dtype=torch.float32).dtype == torch.float32
@@ -390,8 +394,72 @@ class HipOps:
                                             _code(out_dtype), self._stream()), "gemm_nt")
         return y
 
+    # ---- a norm finished inside the products around it (ScaledRows)
+    def can_defer_norm(self, M, w_last, w_first, gated_first):
+        """Whether, for M rows, the product by w_last [H, K1] can add its result into the residual stream
+        and leave the rows of the norm that follows unfinished (linear_add_norm), and the product by
+        w_first ([N, H], or [2N, H] gated) can finish them: both must be products that the sweep forms."""
+        if not self.defer_norms or M < 1 or M > 16:
+            return False
+        for w in (w_last, w_first):
+            if w.dtype != torch.bfloat16 or w.dim() != 2 or w.device != self.device:
+                return False
+        H = w_last.shape[0]
+        if w_first.shape[1] != H or H < self.cu_count or (gated_first and w_first.shape[0] % 2):
+            return False
+        if self.lib.ra_gemm_sweep_workgroups(H, self.cu_count) > 256:      # shares of a row's sum that the next product adds up
+            return False
+        return bool(self.lib.ra_gemm_sweep_fits(M, w_last.shape[1]) and self.lib.ra_gemm_sweep_fits(M, H))
+
+    def _sweep_norm(self, x, w, gated, out_dtype, rows_in=None, h=None, w_next=None):
+        """The sweeping product with a row scale from rows_in (ScaledRows) and, with h, the residual epilogue."""
+        M, K = x.shape
+        N = w.shape[0] // 2 if gated else w.shape[0]
+        if not self.lib.ra_gemm_sweep_fits(M, K) or M > 32:
+            raise KernelError(f"rows with an unfinished norm need the sweeping product, which does not take {M} x {K}")
+        out = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        psq_in = n_in = cols = None
+        eps = 0.0
+        if rows_in is not None:
+            self._want(rows_in.partials, "partial sums of squares", torch.float32, 2)
+            if rows_in.partials.shape[0] != M:
+                raise KernelError(f"partial sums for {rows_in.partials.shape[0]} rows, x has {M}")
+            psq_in, n_in, cols, eps = rows_in.partials, rows_in.partials.shape[1], rows_in.size, rows_in.eps
+        psq_out = None
+        if h is not None:
+            self._want(h, "residual stream", torch.float32, 2)
+            self._want(w_next, "norm weight", torch.float32, 1)
+            if tuple(h.shape) != (M, N) or w_next.shape[0] != N or gated or out_dtype != torch.bfloat16 or M > 16:
+                raise KernelError(f"linear_add_norm: x {tuple(x.shape)}, weight {tuple(w.shape)}, h {tuple(h.shape)}")
+            psq_out = torch.empty(M, self.lib.ra_gemm_sweep_workgroups(N, self.cu_count), dtype=torch.float32,
+                                  device=self.device)
+        self._check(self.lib.ra_gemm_sweep_norm_bf16(
+            _ptr(x), _ptr(w), _ptr(out), M, N, K, 1 if gated else 0, _code(out_dtype), self.cu_count,
+            _ptr(psq_in), n_in or 0, cols or 0, float(eps), _ptr(h), _ptr(w_next), _ptr(psq_out), self._stream()),
+            "gemm_sweep_norm")
+        return out, psq_out
+
+    def linear_add_norm(self, x, w, h, norm_weight, eps):
+        """h += x @ w^T (the result rounded to the compute dtype first, as a stored result would be), and
+        the rows of RMSNorm(h) with this weight and eps left unfinished: ScaledRows for linear() or
+        linear_silu_mul(). x: plain rows or ScaledRows."""
+        rows_in = x if isinstance(x, ScaledRows) else None
+        xt = x.tensor if rows_in is not None else x
+        self._want(xt, "x", torch.bfloat16, 2)
+        self._want(w, "weight", torch.bfloat16, 2)
+        if w.shape[1] != xt.shape[1]:
+            raise KernelError(f"linear_add_norm: x {tuple(xt.shape)} times weight {tuple(w.shape)}^T")
+        xw, psq = self._sweep_norm(xt, w, False, torch.bfloat16, rows_in, h, norm_weight)
+        return ScaledRows(xw, psq, w.shape[0], eps)
+
     def linear(self, x, w, out_dtype=None):
-        """y = x @ w^T, x [M, K], w [N, K]."""
+        """y = x @ w^T, x [M, K] (or ScaledRows: rows whose norm this product finishes), w [N, K]."""
+        if isinstance(x, ScaledRows):
+            self._want(x.tensor, "x", torch.bfloat16, 2)
+            self._want(w, "weight", torch.bfloat16, 2)
+            if w.shape[1] != x.tensor.shape[1]:
+                raise KernelError(f"linear: x {tuple(x.tensor.shape)} times weight {tuple(w.shape)}^T")
+            return self._sweep_norm(x.tensor, w, False, out_dtype or torch.bfloat16, x)[0]
         self._want(x, "x", dims=2)
         self._want(w, "weight", x.dtype, 2)
         M, K = x.shape
@@ -426,6 +494,12 @@ class HipOps:
 
     def linear_silu_mul(self, x, w_gate_up):
         """silu(x @ Wg^T) * (x @ Wu^T) for w_gate_up = [Wg; Wu]: one kernel for few rows, else two."""
+        if isinstance(x, ScaledRows):
+            self._want(x.tensor, "x", torch.bfloat16, 2)
+            self._want(w_gate_up, "gate-up weight", torch.bfloat16, 2)
+            if w_gate_up.shape[1] != x.tensor.shape[1] or w_gate_up.shape[0] % 2:
+                raise KernelError(f"linear_silu_mul: x {tuple(x.tensor.shape)}, weight {tuple(w_gate_up.shape)}")
+            return self._sweep_norm(x.tensor, w_gate_up, True, torch.bfloat16, x)[0]
         self._want(x, "x", dims=2)
         self._want(w_gate_up, "gate-up weight", x.dtype, 2)
         M, K = x.shape

@@ -78,9 +78,16 @@ class Decoder:
         """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
         h = self.embedding.forward(step.token_ids, step)
         pending = None
-        for call in self.schedule:
+        for i, call in enumerate(self.schedule):
             view = cache.view(call.cache) if call.cache is not None else None
-            h, pending = self.blocks[call.block].forward(h, pending, step, view, call.writes_cache)
+            block = self.blocks[call.block]
+            if getattr(block, "first_norm", None) is not None and i + 1 < len(self.schedule):
+                # an arrangement that says what it begins with also takes the block after it, to finish
+                # the norm between the two inside their products where the kernel set can
+                h, pending = block.forward(h, pending, step, view, call.writes_cache,
+                                           next=self.blocks[self.schedule[i + 1].block])
+            else:
+                h, pending = block.forward(h, pending, step, view, call.writes_cache)
         if step.n_logit_rows == 0:
             return None
         x = self.final_norm.forward(h, pending, out_rows=step.logit_rows)

@@ -58,6 +58,10 @@ class PagedAttention:
         self.w_qn = rt.vector32(tensors["q_norm"]) if self.eps is not None else None
         self.w_kn = rt.vector32(tensors["k_norm"]) if self.eps is not None else None
         self._fusable = self.position is None or hasattr(self.position, "tables")
+        # x goes into one product only and the output comes out of one: a norm before may be left to
+        # the first (ScaledRows as x), a norm after may be finished inside the second (sink)
+        self.first_product = (self.w_qkv, False)
+        self.last_product = self.w_o
 
     def cache_spec(self):
         return PagedKVSpec(self.n_kv, self.d, self.window)
@@ -68,8 +72,9 @@ class PagedAttention:
         rows = ops.prefill_tile_rows(self.d, self.rt.dtype) if hasattr(ops, "prefill_tile_rows") else None
         return {"prefill_tile_rows": {rows}} if rows else {}
 
-    def forward(self, x, step, cache, write_cache=True):
+    def forward(self, x, step, cache, write_cache=True, sink=None):
         rt, ops = self.rt, self.rt.ops
+        project = sink.project if sink is not None else ops.linear
         T, Hq, Hkv, D = x.shape[0], self.n_q, self.n_kv, self.d
         tables = step.groups[cache.group]
         qkv = ops.linear(x, self.w_qkv)                              # [T, (Hq+2Hkv)*D]
@@ -80,7 +85,7 @@ class PagedAttention:
             if ops.attention_qkv(qkv, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale,
                                  int(self.window) if self.window else 0, Hq, Hkv, D, self.w_qn, self.w_kn,
                                  float(self.eps) if self.eps is not None else 0.0, cos, sin, rot):
-                return ops.linear(o.view(T, Hq * D), self.w_o)
+                return project(o.view(T, Hq * D), self.w_o)
         q = rt.empty(T, Hq, D)
         if self._fusable:
             cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
@@ -103,7 +108,7 @@ class PagedAttention:
         o = rt.empty(T, Hq, D)
         ops.attention(q, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale,
                       int(self.window) if self.window else 0)
-        return ops.linear(o.view(T, Hq * D), self.w_o)
+        return project(o.view(T, Hq * D), self.w_o)
 
 
 register_part("mixer", "attention", PagedAttention)

@@ -26,11 +26,13 @@ class SwiGLU:
         self.w_gate_up = rt.product(torch.cat([rt.matrix(tensors["gate_proj"]), rt.matrix(tensors["up_proj"])],
                                               dim=0).contiguous(), gated=True)
         self.w_down = rt.product(rt.matrix(tensors["down_proj"]))
+        self.first_product = (self.w_gate_up, True)        # (see PagedAttention)
+        self.last_product = self.w_down
 
-    def forward(self, x, step=None):
+    def forward(self, x, step=None, sink=None):
         ops = self.rt.ops
         a = ops.linear_silu_mul(x, self.w_gate_up)         # [T, I] = silu(gate) * up, gate rows first
-        return ops.linear(a, self.w_down)
+        return sink.project(a, self.w_down) if sink is not None else ops.linear(a, self.w_down)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

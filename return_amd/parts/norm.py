@@ -7,6 +7,7 @@ offset 0.0 (rollout/monkey_patch/qwen3.py:15-17).
 from __future__ import annotations
 
 from .registry import register_part
+from .runtime import ScaledRows
 
 
 class RMSNorm:
@@ -28,6 +29,12 @@ class RMSNorm:
 
     def forward(self, h, delta=None, out_rows=None):
         """h (fp32 [T, size]) += delta in place; returns norm(h) (only rows out_rows, if given)."""
+        if isinstance(delta, ScaledRows):
+            # the product before has added its result into h and left this norm's rows unfinished:
+            # the next product applies 1/rms itself
+            if delta.norm is not self or out_rows is not None:
+                raise ValueError("rows prepared for another norm, or for all rows where some are wanted")
+            return delta
         rows = h.shape[0] if out_rows is None else out_rows.shape[0]
         out = self.rt.empty(rows, self.size)
         self.rt.ops.add_rmsnorm(h, delta, self.weight, self.eps, out, out_rows)

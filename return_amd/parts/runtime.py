@@ -8,6 +8,42 @@ import torch
 _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
+class ScaledRows:
+    """Rows whose RMSNorm is not finished: ``tensor`` [M, size] holds h * w_norm in the compute dtype,
+    ``partials`` [M, n] fp32 hold shares of each row's sum of squares of h. The norm's 1/rms is a
+    number per row, so a product may multiply its result rows by rsqrt(sum(partials) / size + eps)
+    instead of its operand: norm(h) W^T = rstd * ((h * w_norm) W^T). A kernel set that offers
+    ``linear_add_norm`` makes such rows in the epilogue of the product that feeds the residual
+    stream, and takes them in ``linear`` and ``linear_silu_mul``; ``norm`` is the norm part they
+    were made for, which hands them on as its output."""
+    __slots__ = ("tensor", "partials", "size", "eps", "norm")
+
+    def __init__(self, tensor, partials, size, eps, norm=None):
+        self.tensor, self.partials, self.size, self.eps, self.norm = tensor, partials, int(size), float(eps), norm
+
+    @property
+    def shape(self):
+        return self.tensor.shape
+
+    @property
+    def dtype(self):
+        return self.tensor.dtype
+
+
+class NormSink:
+    """Given to a part whose last product feeds the residual stream when the kernel set can finish
+    the step's next norm inside that product: ``project(x, w)`` adds x @ w^T into ``h`` and returns
+    the next part's input as ScaledRows, in place of the plain product that the next norm would add."""
+
+    def __init__(self, ops, h, norm):
+        self.ops, self.h, self.norm = ops, h, norm
+
+    def project(self, x, w):
+        rows = self.ops.linear_add_norm(x, w, self.h, self.norm.weight, self.norm.eps)
+        rows.norm = self.norm
+        return rows
+
+
 class Runtime:
     """Device, compute dtype and kernel set of one engine.
 

@@ -6,7 +6,7 @@ import torch
 
 from return_amd import SamplingParams
 from return_amd.config import EngineConfig
-from return_amd.engine import Engine, ModelRunner
+from return_amd.engine import Engine, ModelRunner, StepEntry
 from tests import trace_tools as tt
 from tests.conftest import TINY_A, TINY_B
 from tests.plain import qwen3_plain as plain
@@ -371,3 +371,43 @@ def test_duty_and_decode_streak(folder_a):
     assert 0 < st["decode_duty"] < 1 and 0 < st["prefill_duty"] < 1
     assert st["decode_duty"] + st["prefill_duty"] <= 1.0 + 1e-9
     assert abs(st["decode_duty"] * st["run_seconds"] - eng.decode_seconds) < 1e-6
+
+
+def test_norms_are_finished_inside_the_products_in_steps_of_few_rows(folder_b):
+    """A step of up to 16 rows leaves every norm between two products to those products (the kernel
+    set's linear_add_norm, and ScaledRows into linear / linear_silu_mul); a step of more rows, the first
+    norm of the first layer and the last norm (on the wanted rows only) run as norms of their own. The
+    logits are the plain implementation's either way."""
+    from return_amd.parts.runtime import ScaledRows
+    cfg, w = plain.read_folder(folder_b)
+    L = cfg["num_hidden_layers"]
+    toks = tt.random_tokens(TINY_B["vocab_size"], 40, seed=3)
+    want = plain.logits(cfg, w, toks)
+    for defer in (True, False):
+        runner = runner_for(folder_b, 128, defer_norms=defer)
+        ops = runner.rt.ops
+        calls = {"add_norm": 0, "scaled_in": 0, "norm": 0}
+        for name, key in (("linear_add_norm", "add_norm"), ("add_rmsnorm", "norm")):
+            def counted(*a, _f=getattr(ops, name), _k=key, **k):
+                calls[_k] += 1
+                return _f(*a, **k)
+            setattr(ops, name, counted)
+        for name in ("linear", "linear_silu_mul"):
+            def counted(x, *a, _f=getattr(ops, name), **k):
+                calls["scaled_in"] += isinstance(x, ScaledRows)
+                return _f(x, *a, **k)
+            setattr(ops, name, counted)
+        if not defer:
+            ops.can_defer_norm = lambda *a: False
+        runner.add_request("r")
+        got = [runner.step([StepEntry("r", toks[:24], list(range(24)))])]          # 24 rows: norms of their own
+        assert calls == {"add_norm": 0, "scaled_in": 0, "norm": 2 * L + 1}
+        calls.update(add_norm=0, scaled_in=0, norm=0)
+        got.append(runner.step([StepEntry("r", toks[24:], list(range(16)))]))     # 16 rows
+        if defer:
+            # every layer's two norms but the very first are left to the products; the last norm stands alone
+            # (the stand-in's gated product calls its plain one, so each of the L gated products counts twice)
+            assert calls == {"add_norm": 2 * L - 1, "scaled_in": 2 * L - 1 + L, "norm": 2}
+        else:
+            assert calls == {"add_norm": 0, "scaled_in": 0, "norm": 2 * L + 1}
+        torch.testing.assert_close(torch.cat(got).cpu(), want, atol=2e-4, rtol=2e-4)

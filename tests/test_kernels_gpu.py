@@ -295,6 +295,59 @@ def test_every_way_to_form_a_product(ops, monkeypatch, N, K):
             "gated resident512", "gated sweep"} <= ways
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("H,K1,N2", [(512, 264, 331), (4096, 4096, 1000), (1024, 12288, 760), (264, 520, 4500)])
+def test_norm_finished_inside_the_products_around_it(ops, ref, M, H, K1, N2):
+    """h += x W1^T inside the product, the rows of the norm that follows left unfinished, and the
+    products after it that finish them (plain, fp32 results, gated): against the residual addition,
+    the norm and the products one after the other. K1 within one span of the sweep and beyond it, a
+    width that is no multiple of the workgroups, more and fewer columns than workgroups."""
+    from return_amd.parts.runtime import ScaledRows
+    x = rnd(M, K1, dtype=torch.bfloat16, seed=1)
+    w1 = rnd(H, K1, dtype=torch.bfloat16, seed=2, scale=0.05)
+    w2 = rnd(2 * N2, H, dtype=torch.bfloat16, seed=3, scale=0.05)
+    wn = 1.0 + 0.2 * rnd(H, seed=4)
+    h0 = rnd(M, H, seed=5, scale=2.0)
+    eps = 1e-5
+    assert ops.can_defer_norm(M, w1, w2, True) and ops.can_defer_norm(M, w1, w2, False)
+    h = h0.clone()
+    rows = ops.linear_add_norm(x, w1, h, wn, eps)
+    assert isinstance(rows, ScaledRows) and rows.partials.shape[0] == M and rows.size == H
+    # the residual stream: h0 + bf16(x W1^T)
+    delta = (x.double() @ w1.double().t())
+    torch.testing.assert_close(h.double(), h0.double() + delta, atol=2e-2, rtol=2e-2)
+    want_h = h.double()                                     # from here on with the h the kernel made
+    torch.testing.assert_close(rows.tensor.float(), (want_h * wn.double()).float(), **tol(torch.bfloat16))
+    torch.testing.assert_close(rows.partials.double().sum(-1), (want_h * want_h).sum(-1), atol=1e-3, rtol=1e-4)
+    xn = want_h * (1.0 / torch.sqrt((want_h * want_h).mean(-1, keepdim=True) + eps)) * wn.double()
+    torch.testing.assert_close(ops.linear(rows, w2).float(), (xn @ w2.double().t()).float(), **tol(torch.bfloat16))
+    # the products after it, exactly: from the operand as the kernel left it (rounded to bfloat16)
+    xn = rows.tensor.double() * (1.0 / torch.sqrt((want_h * want_h).mean(-1, keepdim=True) + eps))
+    y = xn @ w2.double().t()
+    torch.testing.assert_close(ops.linear(rows, w2).float(), y.float(), **tol(torch.bfloat16))
+    torch.testing.assert_close(ops.linear(rows, w2, out_dtype=torch.float32).double(), y, atol=3e-2, rtol=2e-2)
+    g, u = y[:, :N2], y[:, N2:]
+    torch.testing.assert_close(ops.linear_silu_mul(rows, w2).float(), (g * torch.sigmoid(g) * u).float(),
+                               **tol(torch.bfloat16))
+    # and a second residual product on unfinished rows (x itself ScaledRows)
+    w3 = rnd(H, H, dtype=torch.bfloat16, seed=6, scale=0.05)
+    h2 = h.clone()
+    rows2 = ops.linear_add_norm(rows, w3, h2, wn, eps)
+    torch.testing.assert_close(h2.double(), want_h + xn @ w3.double().t(), atol=3e-2, rtol=2e-2)
+    assert rows2.tensor.shape == (M, H)
+
+
+def test_norms_are_not_deferred_where_the_sweep_does_not_form_the_products(ops):
+    bf = torch.bfloat16
+    w1, w2 = rnd(512, 264, dtype=bf), rnd(300, 512, dtype=bf)
+    assert ops.can_defer_norm(16, w1, w2, False)
+    assert not ops.can_defer_norm(17, w1, w2, False)                    # more rows than the residual epilogue takes
+    assert not ops.can_defer_norm(4, rnd(512, 260, dtype=bf), w2, False)   # K no multiple of 8
+    assert not ops.can_defer_norm(4, w1.float(), w2.float(), False)     # float32: the plain kernels
+    assert not ops.can_defer_norm(4, rnd(100, 264, dtype=bf), rnd(300, 100, dtype=bf), False)   # narrower than the chip
+    assert not ops.can_defer_norm(4, w1, rnd(300, 520, dtype=bf), False)   # widths that do not meet
+
+
 def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
     """tune_products measures every shape at every row count up to the limit, once in a process, and
     notes only ways that exist; a measured choice is what route_* returns from then on; a kernel

@@ -10,6 +10,8 @@ from __future__ import annotations
 
 import torch
 
+from return_amd.parts.runtime import ScaledRows
+
 
 class TorchOps:
     def __init__(self, device="cpu"):
@@ -97,12 +99,34 @@ class TorchOps:
 
     # rollout/monkey_patch/qwen3.py:21 (F.linear)
     def linear(self, x, w, out_dtype=None):
+        if isinstance(x, ScaledRows):                       # rows whose norm this product finishes
+            y = (x.tensor.float() @ w.float().t()) * self._rstd(x)
+            return y.to(out_dtype or x.tensor.dtype)
         return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
+
+    # A norm finished inside the products around it, as HipOps offers for steps of few rows
+    # (norm(h) W^T = rstd * ((h * w_norm) W^T), rollout/fused.py:6-17): here for up to 16 rows of any
+    # dtype, with the sum of squares in SHARES columns so that the adding-up is exercised too.
+    SHARES = 3
+
+    @staticmethod
+    def _rstd(rows):
+        return 1.0 / torch.sqrt(rows.partials.sum(-1, keepdim=True) / rows.size + rows.eps)
+
+    def can_defer_norm(self, M, w_last, w_first, gated_first):
+        return 1 <= M <= 16 and w_first.shape[1] == w_last.shape[0] >= self.SHARES
+
+    def linear_add_norm(self, x, w, h, norm_weight, eps):
+        y = self.linear(x, w)                               # (rounded to the compute dtype like a stored result)
+        h += y.float()
+        sq = h * h
+        cut = [sq[:, i::self.SHARES].sum(-1) for i in range(self.SHARES)]
+        return ScaledRows((h * norm_weight).to(y.dtype), torch.stack(cut, dim=1), h.shape[1], eps)
 
     # rollout/monkey_patch/qwen3.py:20-22
     def linear_silu_mul(self, x, w_gate_up):
         gu = self.linear(x, w_gate_up)
-        out = torch.empty(x.shape[0], w_gate_up.shape[0] // 2, dtype=x.dtype, device=x.device)
+        out = torch.empty(gu.shape[0], w_gate_up.shape[0] // 2, dtype=gu.dtype, device=gu.device)
         self.silu_mul(gu, out)
         return out
 
