@@ -146,6 +146,113 @@ extern "C" int ra_add_rmsnorm(float* h, const void* delta, const float* w, float
     return ra_launch_status();
 }
 
+// The same where the part before left its result as n_slabs 32-bit shares [n_slabs, rows of h, H] (a
+// product whose K was cut into pieces, one share each): delta = their sum in slab order, rounded to T
+// as the one product's stored result would have been.
+template <typename T>
+__global__ void add_slabs_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ slabs, int n_slabs,
+                                         size_t slab_stride, const float* __restrict__ w, float eps,
+                                         T* __restrict__ out, const int* __restrict__ rows, int H) {
+    __shared__ float scratch[16];
+    const int m = blockIdx.x;
+    const size_t r = rows ? (size_t)rows[m] : (size_t)m;
+    float* hr = h + r * H;
+    const float* sr = slabs + r * H;
+    const bool write_back = rows == nullptr;
+    auto delta_at = [&](int c) {
+        float d = 0.f;
+        for (int s = 0; s < n_slabs; ++s) d += sr[(size_t)s * slab_stride + c];
+        return round_to<T>(d);
+    };
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float v = hr[c] + delta_at(c);
+        if (write_back) hr[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    T* o = out + (size_t)m * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = hr[c];                       // same thread wrote it above
+        if (!write_back) v += delta_at(c);
+        o[c] = from_f<T>(v * rstd * w[c]);
+    }
+}
+
+// The same for H % 4 == 0, H <= 4096 and S shares known at compile time: 16-byte accesses, every load of
+// a thread asked for at once, the row kept in registers between the two phases. 1024 threads a row.
+template <typename T, int S>
+__global__ __launch_bounds__(1024) void add_slabs_rmsnorm_vec_kernel(
+    float* __restrict__ h, const float* __restrict__ slabs, size_t slab_stride, const float* __restrict__ w, float eps,
+    T* __restrict__ out, const int* __restrict__ rows, int H) {
+    __shared__ float scratch[16];
+    const int m = blockIdx.x, c = threadIdx.x;
+    const size_t r = rows ? (size_t)rows[m] : (size_t)m;
+    const bool in = c < (H >> 2);
+    const int cc = in ? c : 0;
+    float4 v = reinterpret_cast<const float4*>(h + r * H)[cc];
+    float4 sh[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) sh[s] = reinterpret_cast<const float4*>(slabs + (size_t)s * slab_stride + r * H)[cc];
+    const float4 ww = reinterpret_cast<const float4*>(w)[cc];
+    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int s = 0; s < S; ++s) { d.x += sh[s].x; d.y += sh[s].y; d.z += sh[s].z; d.w += sh[s].w; }
+    v.x += round_to<T>(d.x); v.y += round_to<T>(d.y); v.z += round_to<T>(d.z); v.w += round_to<T>(d.w);
+    if (in && rows == nullptr) reinterpret_cast<float4*>(h + r * H)[c] = v;
+    float ss = in ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f;
+    ss = block_sum(ss, scratch);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    if (in) {
+        T* o = out + (size_t)m * H + 4 * c;
+        const float a = v.x * rstd * ww.x, b = v.y * rstd * ww.y, e = v.z * rstd * ww.z, f = v.w * rstd * ww.w;
+        if constexpr (sizeof(T) == 2) {
+            uint2 p;
+            p.x = (uint32_t)f2bf_bits(a) | ((uint32_t)f2bf_bits(b) << 16);
+            p.y = (uint32_t)f2bf_bits(e) | ((uint32_t)f2bf_bits(f) << 16);
+            *reinterpret_cast<uint2*>(o) = p;
+        } else {
+            *reinterpret_cast<float4*>(o) = make_float4(a, b, e, f);
+        }
+    }
+}
+
+template <typename T>
+static bool launch_slabs_vec(int n_slabs, dim3 grid, hipStream_t st, float* h, const float* slabs, size_t stride,
+                             const float* w, float eps, T* out, const int* rows, int H) {
+    switch (n_slabs) {
+        case 2: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 2>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
+        case 4: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 4>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
+        case 8: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 8>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
+        default: return false;
+    }
+}
+
+// slabs: fp32 [n_slabs, R, H] with R rows as h has them (slab_rows = R).
+extern "C" int ra_add_slabs_rmsnorm(float* h, const float* slabs, int n_slabs, long long slab_rows, const float* w,
+                                    float eps, void* out, const int* rows, int M, int H, int dtype, void* stream) {
+    if (M <= 0) return RA_OK;
+    if (n_slabs <= 0 || slab_rows <= 0 || H <= 0) return RA_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const size_t stride = (size_t)slab_rows * H;
+    dim3 grid(M);
+    if (H % 4 == 0 && H <= 4096) {
+        const bool done = dtype == RA_DTYPE_F32
+            ? launch_slabs_vec<float>(n_slabs, grid, st, h, slabs, stride, w, eps, (float*)out, rows, H)
+            : launch_slabs_vec<bf16>(n_slabs, grid, st, h, slabs, stride, w, eps, (bf16*)out, rows, H);
+        if (done) return ra_launch_status();
+    }
+    dim3 block(H >= 2048 ? 1024 : 256);
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(add_slabs_rmsnorm_kernel<float>, grid, block, 0, st, h, slabs, n_slabs, stride, w, eps,
+                           (float*)out, rows, H);
+    else
+        hipLaunchKernelGGL(add_slabs_rmsnorm_kernel<bf16>, grid, block, 0, st, h, slabs, n_slabs, stride, w, eps,
+                           (bf16*)out, rows, H);
+    return ra_launch_status();
+}
+
 // ------------------------------------------------------------------ residual add alone
 template <typename T>
 __global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__ delta, size_t n) {

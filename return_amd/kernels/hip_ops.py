@@ -12,7 +12,7 @@ from typing import Optional
 
 import torch
 
-from ..parts.runtime import ScaledRows
+from ..parts.runtime import ScaledRows, Slabs
 from . import build as _build
 
 _F32, _BF16 = 0, 1
@@ -52,6 +52,7 @@ def _declare(lib):
     sigs = {
         "ra_embed": [P, P, P, I, I, I, I, P],
         "ra_add_rmsnorm": [P, P, P, F, P, P, I, I, I, P],
+        "ra_add_slabs_rmsnorm": [P, P, I, L, P, F, P, P, I, I, I, P],
         "ra_residual_add": [P, P, L, I, P],
         "ra_head_rmsnorm": [P, P, F, L, I, I, P],
         "ra_rope": [P, P, P, P, I, I, I, I, I, P],
@@ -120,6 +121,11 @@ class HipOps:
             self._library_fp32_out = torch.mm(a, a.t(), out_dtype=torch.float32).dtype == torch.float32
         except (TypeError, RuntimeError):
             self._library_fp32_out = False
+        try:                                 # and the same for a batch of products
+            a = torch.ones(2, 1, 8, dtype=torch.bfloat16, device=self.device)
+            self._library_bmm_fp32 = torch.bmm(a, a.transpose(1, 2), out_dtype=torch.float32).dtype == torch.float32
+        except (TypeError, RuntimeError):
+            self._library_bmm_fp32 = False
         # whether the library's float32 product is a true 32-bit one (against a 64-bit product; operands
         # rounded to a shorter mantissa would be off by 1e-3)
         g = torch.Generator(device="cpu").manual_seed(0)
@@ -207,6 +213,19 @@ class HipOps:
         R, H = h.shape
         if weight.shape[0] != H or out.shape[1] != H:
             raise KernelError(f"add_rmsnorm: h {tuple(h.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+        if isinstance(delta, Slabs):
+            self._want(delta.tensor, "shares of the product", torch.float32, 3)
+            if tuple(delta.tensor.shape[1:]) != (R, H):
+                raise KernelError(f"add_rmsnorm: shares {tuple(delta.tensor.shape)} do not match h {tuple(h.shape)}")
+            if rows is not None:
+                self._want(rows, "row list", torch.int32, 1)
+            M = R if rows is None else rows.shape[0]
+            if out.shape[0] != M:
+                raise KernelError(f"add_rmsnorm: out has {out.shape[0]} rows, {M} wanted")
+            self._check(self.lib.ra_add_slabs_rmsnorm(_ptr(h), _ptr(delta.tensor), delta.tensor.shape[0], R, _ptr(weight),
+                                                      float(eps), _ptr(out), _ptr(rows), M, H, _code(out.dtype),
+                                                      self._stream()), "add_slabs_rmsnorm")
+            return
         if delta is not None:
             self._want(delta, "delta", out.dtype, 2)
             if tuple(delta.shape) != (R, H):
@@ -342,11 +361,22 @@ class HipOps:
                 return r
         return 0                                          # more rows than are ever measured: the library
 
+    SPLITS = (2, 4, 8)            # pieces of K that a product for the residual stream may be cut into
+
     def route_linear(self, M, N, K, out_dtype):
-        """How linear() forms a bfloat16 product of M rows: the measured choice if there is one, else the rule."""
+        """How linear() forms a bfloat16 product of M rows: the measured choice if there is one, else the rule.
+        out_dtype "residual": the product whose result goes into the residual stream (linear_residual), bfloat16
+        rows or, "split<n>", n shares of 32-bit sums from the library's batched product over n pieces of K."""
         hit = self.product_plan.get((self._rows_step(M), N, K, False, out_dtype))
         if hit is not None:
             return hit
+        if out_dtype == "residual":
+            # measured on MI355X (8B shape, down: N 4,096, K 12,288): at 17 to 64 rows the library gives one
+            # workgroup to each tile of the result and leaves half the chip idle; four pieces of K as a
+            # batch take 24 µs against 29 to 38
+            if 16 < M <= 64 and K >= 8192 and N * 2 <= K and K % 32 == 0 and self._library_bmm_fp32:
+                return "split4"
+            out_dtype = torch.bfloat16
         if out_dtype in (torch.bfloat16, torch.float32) and self.use_sweep(M, N, K, False):
             return "sweep"
         if out_dtype in (torch.bfloat16, torch.float32) and self.use_resident(M, N, K, False):
@@ -452,6 +482,32 @@ class HipOps:
         xw, psq = self._sweep_norm(xt, w, False, torch.bfloat16, rows_in, h, norm_weight)
         return ScaledRows(xw, psq, w.shape[0], eps)
 
+    def _split_product(self, x, w, pieces):
+        """x @ w^T as `pieces` shares [pieces, M, N] fp32, share i from columns i*K/pieces .. of K: one batched
+        library product over strided views of x and w (nothing is copied)."""
+        M, K = x.shape
+        N = w.shape[0]
+        xs = x.view(M, pieces, K // pieces).transpose(0, 1)
+        wv = w.view(N, pieces, K // pieces).permute(1, 2, 0)
+        return Slabs(torch.bmm(xs, wv, out_dtype=torch.float32))
+
+    def linear_residual(self, x, w):
+        """x @ w^T for the residual stream: bfloat16 (or float32) rows as linear() gives them, or Slabs
+        where cutting K into pieces is faster; what takes the result must take both (the norm part does)."""
+        if isinstance(x, ScaledRows) or x.dtype != torch.bfloat16:
+            return self.linear(x, w)
+        self._want(x, "x", dims=2)
+        self._want(w, "weight", x.dtype, 2)
+        M, K = x.shape
+        if w.shape[1] != K:
+            raise KernelError(f"linear: x {tuple(x.shape)} times weight {tuple(w.shape)}^T")
+        if M == 0:
+            return self.linear(x, w)
+        how = self.route_linear(M, w.shape[0], K, "residual")
+        if how.startswith("split"):
+            return self._split_product(x, w, int(how[5:]))
+        return self._linear_by(how, x, w, torch.bfloat16)
+
     def linear(self, x, w, out_dtype=None):
         """y = x @ w^T, x [M, K] (or ScaledRows: rows whose norm this product finishes), w [N, K]."""
         if isinstance(x, ScaledRows):
@@ -511,6 +567,9 @@ class HipOps:
 
     def _candidates(self, M, N, K, gated, out_dtype):
         """The ways that can form this product at all."""
+        residual = out_dtype == "residual"
+        if residual:
+            out_dtype = torch.bfloat16
         if gated:
             c = ["two"]
             if M <= 16 and K % 8 == 0:
@@ -523,6 +582,8 @@ class HipOps:
             c += ["resident256", "resident512"]
         if self.lib.ra_gemm_sweep_fits(M, K):
             c.append("sweep")
+        if residual and self._library_bmm_fp32 and M > 16:
+            c += [f"split{n}" for n in self.SPLITS if K % (8 * n) == 0]
         return c
 
     def tune_products(self, products, max_rows=64, margin=0.93):
@@ -567,9 +628,17 @@ class HipOps:
             x = torch.randn(rows, K, device=self.device, dtype=torch.float32).to(torch.bfloat16)
             times = {}
             for how in cands:
-                run = (lambda w, how=how: self._gated_by(how, x, w)) if gated else \
-                      (lambda w, how=how: self._linear_by(how, x, w, out_dtype))
+                if gated:
+                    run = lambda w, how=how: self._gated_by(how, x, w)
+                elif how.startswith("split"):
+                    run = lambda w, how=how: self._split_product(x, w, int(how[5:]))
+                else:
+                    run = lambda w, how=how: self._linear_by(how, x, w, torch.bfloat16 if out_dtype == "residual" else out_dtype)
                 times[how] = self._time_over(run, weights, launches)
+                if how.startswith("split"):
+                    # what the norm after it pays for reading the shares instead of one result (it runs one
+                    # workgroup a row; measured on MI355X at 64 rows of 4,096: 4 shares 3 µs, 8 shares 6.5 µs)
+                    times[how] += int(how[5:]) * rows * N * 4 / 1.5e12
         finally:
             self.product_plan = saved
         best = min(times, key=times.get)

@@ -81,11 +81,17 @@ class Decoder:
         for i, call in enumerate(self.schedule):
             view = cache.view(call.cache) if call.cache is not None else None
             block = self.blocks[call.block]
-            if getattr(block, "first_norm", None) is not None and i + 1 < len(self.schedule):
-                # an arrangement that says what it begins with also takes the block after it, to finish
-                # the norm between the two inside their products where the kernel set can
-                h, pending = block.forward(h, pending, step, view, call.writes_cache,
-                                           next=self.blocks[self.schedule[i + 1].block])
+            if getattr(block, "first_norm", None) is not None:
+                # an arrangement that says what it begins with is also told what takes its output: the
+                # next block's first norm and first product (which may finish that norm between them),
+                # or the last norm (which runs on the wanted rows only, as a kernel of its own)
+                if i + 1 < len(self.schedule):
+                    nxt = self.blocks[self.schedule[i + 1].block]
+                    after = (nxt.first_norm, getattr(nxt, "first_product", None)) \
+                        if getattr(nxt, "first_norm", None) is not None else None
+                else:
+                    after = (self.final_norm, None)
+                h, pending = block.forward(h, pending, step, view, call.writes_cache, after=after)
             else:
                 h, pending = block.forward(h, pending, step, view, call.writes_cache)
         if step.n_logit_rows == 0:

@@ -54,7 +54,7 @@ class PagedAttention:
             raise KeyError(f"attention names position encoding {params['position']!r}, which the model lacks")
         self.w_qkv = rt.product(torch.cat([rt.matrix(tensors["q_proj"]), rt.matrix(tensors["k_proj"]),
                                            rt.matrix(tensors["v_proj"])], dim=0).contiguous())
-        self.w_o = rt.product(rt.matrix(tensors["o_proj"]))
+        self.w_o = rt.product(rt.matrix(tensors["o_proj"]), residual=True)
         self.w_qn = rt.vector32(tensors["q_norm"]) if self.eps is not None else None
         self.w_kn = rt.vector32(tensors["k_norm"]) if self.eps is not None else None
         self._fusable = self.position is None or hasattr(self.position, "tables")

@@ -12,28 +12,32 @@ An arrangement is a class with
     forward(self, h, pending, step, cache, write_cache) -> (h, pending)
         h: fp32 residual stream [T, H]; pending: the last part's output, not yet added to h
         (or None); cache: the cache manager's view for this call's cache layer (or None).
-    Optional: first_norm / first_product attributes and a next= argument of forward (see PreNormBlock),
+    Optional: first_norm / first_product attributes and an after= argument of forward (see PreNormBlock),
     with which the norm between two blocks can be finished inside their products.
 It is registered with register_arrangement(name, cls) and named in BlockSpec.arrangement.
 """
 from __future__ import annotations
 
-from .runtime import NormSink
+from .runtime import NormSink, ResidualSink
 
 
 def norm_sink(h, producer, norm, consumer_first_product):
-    """A NormSink for the norm between two parts, or None: when the producer ends in one product and
-    the consumer begins with one (their last_product / first_product attributes), the norm is a plain
-    RMSNorm part, and the kernel set says that it can finish the norm inside these two products for
-    this many rows (can_defer_norm)."""
+    """The sink for the last product of ``producer``, whose result goes through ``norm`` into the next
+    part, or None. A NormSink when the producer ends in one product and the consumer begins with one
+    (their last_product / first_product attributes), the norm is a plain RMSNorm part, and the kernel
+    set says that it can finish the norm inside these two products for this many rows
+    (can_defer_norm); else a ResidualSink when the norm takes a product's result in every form
+    (takes_slabs); else None: the part forms its product as it does for anyone."""
     ops = getattr(getattr(norm, "rt", None), "ops", None)
     last = getattr(producer, "last_product", None)
-    if last is None or consumer_first_product is None or not hasattr(ops, "can_defer_norm"):
+    if last is None or ops is None or norm is None:
         return None
-    if not (hasattr(norm, "weight") and hasattr(norm, "eps")):
-        return None
-    first, gated = consumer_first_product
-    return NormSink(ops, h, norm) if ops.can_defer_norm(h.shape[0], last, first, gated) else None
+    if consumer_first_product is not None and hasattr(ops, "can_defer_norm") and \
+            hasattr(norm, "weight") and hasattr(norm, "eps"):
+        first, gated = consumer_first_product
+        if ops.can_defer_norm(h.shape[0], last, first, gated):
+            return NormSink(ops, h, norm)
+    return ResidualSink(ops) if getattr(norm, "takes_slabs", False) else None
 
 
 class PreNormBlock:
@@ -52,18 +56,17 @@ class PreNormBlock:
     def step_needs(self):
         return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
 
-    def forward(self, h, pending, step, cache, write_cache=True, next=None):
+    def forward(self, h, pending, step, cache, write_cache=True, after=None):
         """h: fp32 residual; pending: output of the last part, not yet added. Returns (h, pending).
-        next: the block that runs after this one (None after the last): the norm it begins with may be
-        finished inside this block's last product and its first one."""
+        after: (norm, first product) of what takes this block's pending output, the next block's
+        first_norm and first_product or the model's last norm and None; None: unknown. The norm may be
+        finished inside this block's last product and that first one, or take the product in shares."""
         x = self.mixer_norm.forward(h, pending)
         sink = norm_sink(h, self.mixer, self.feed_forward_norm, getattr(self.feed_forward, "first_product", None))
         a = self.mixer.forward(x, step, cache, write_cache, sink) if sink is not None else \
             self.mixer.forward(x, step, cache, write_cache)
         x = self.feed_forward_norm.forward(h, a)
-        sink = None
-        if next is not None and getattr(next, "first_norm", None) is not None:
-            sink = norm_sink(h, self.feed_forward, next.first_norm, getattr(next, "first_product", None))
+        sink = norm_sink(h, self.feed_forward, after[0], after[1]) if after is not None else None
         f = self.feed_forward.forward(x, step, sink) if sink is not None else self.feed_forward.forward(x, step)
         return h, f
 

@@ -25,7 +25,7 @@ class SwiGLU:
         self.inter = int(params["intermediate_size"])
         self.w_gate_up = rt.product(torch.cat([rt.matrix(tensors["gate_proj"]), rt.matrix(tensors["up_proj"])],
                                               dim=0).contiguous(), gated=True)
-        self.w_down = rt.product(rt.matrix(tensors["down_proj"]))
+        self.w_down = rt.product(rt.matrix(tensors["down_proj"]), residual=True)
         self.first_product = (self.w_gate_up, True)        # (see PagedAttention)
         self.last_product = self.w_down
 

@@ -11,6 +11,8 @@ from .runtime import ScaledRows
 
 
 class RMSNorm:
+    takes_slabs = True          # forward's delta may be Slabs (the kernel set's add_rmsnorm adds them up)
+
     @staticmethod
     def tensor_shapes(params):
         return {"weight": (params["size"],)}

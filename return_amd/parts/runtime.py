@@ -30,10 +30,39 @@ class ScaledRows:
         return self.tensor.dtype
 
 
-class NormSink:
-    """Given to a part whose last product feeds the residual stream when the kernel set can finish
-    the step's next norm inside that product: ``project(x, w)`` adds x @ w^T into ``h`` and returns
-    the next part's input as ScaledRows, in place of the plain product that the next norm would add."""
+class Slabs:
+    """A product's result left as shares: ``tensor`` [n, M, N] fp32, the result being their sum in order
+    (a product whose K was cut into n pieces, one share each). A norm that takes them adds them up,
+    rounds the sum as the one product's result would have been rounded, and adds it into the residual
+    stream."""
+    __slots__ = ("tensor",)
+
+    def __init__(self, tensor):
+        self.tensor = tensor
+
+    @property
+    def shape(self):
+        return self.tensor.shape[1:]
+
+
+class ResidualSink:
+    """Given to a part for its last product when what the product makes goes nowhere but into the
+    residual stream, through a norm that takes every form of it: ``project(x, w)`` is x @ w^T in
+    whichever form the kernel set forms fastest for that (``linear_residual``: plain rows or Slabs)."""
+
+    def __init__(self, ops):
+        self.ops = ops
+
+    def project(self, x, w):
+        if hasattr(self.ops, "linear_residual"):
+            return self.ops.linear_residual(x, w)
+        return self.ops.linear(x, w)
+
+
+class NormSink(ResidualSink):
+    """The sink when the kernel set can finish the step's next norm inside the product: ``project(x, w)``
+    adds x @ w^T into ``h`` and returns the next part's input as ScaledRows, in place of the product's
+    result that the next norm would add."""
 
     def __init__(self, ops, h, norm):
         self.ops, self.h, self.norm = ops, h, norm
@@ -80,11 +109,13 @@ class Runtime:
             self._cast[key] = hit
         return hit[1]
 
-    def product(self, w: torch.Tensor, gated: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        """Notes that the part will multiply by w (ops.linear, or ops.linear_silu_mul when gated) and
-        returns w. The kernel set may measure, once the model is built, which of its ways to form the
-        products of these shapes is fastest; a part that does not note its weights is served by rules."""
-        self.products.append((w, gated, out_dtype))
+    def product(self, w: torch.Tensor, gated: bool = False, out_dtype: Optional[torch.dtype] = None,
+                residual: bool = False) -> torch.Tensor:
+        """Notes that the part will multiply by w (ops.linear, or ops.linear_silu_mul when gated; residual:
+        through a sink, as the product whose result goes into the residual stream) and returns w. The
+        kernel set may measure, once the model is built, which of its ways to form the products of these
+        shapes is fastest; a part that does not note its weights is served by rules."""
+        self.products.append((w, gated, "residual" if residual else out_dtype))
         return w
 
     def vector32(self, t: torch.Tensor) -> torch.Tensor:

@@ -337,6 +337,55 @@ def test_norm_finished_inside_the_products_around_it(ops, ref, M, H, K1, N2):
     assert rows2.tensor.shape == (M, H)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("R,H,S", [(5, 120, 2), (33, 1000, 4), (64, 4096, 8)])
+def test_add_rmsnorm_takes_a_product_in_shares(ops, ref, dtype, R, H, S):
+    """The norm adds the shares of a product up in order, rounds the sum as the one product's result
+    would have been rounded, and goes on as with that result; all rows, and a list of rows."""
+    from return_amd.parts.runtime import Slabs
+    shares = Slabs(rnd(S, R, H, seed=8))
+    total = torch.zeros(R, H, device=DEV)
+    for i in range(S):                                      # in order, as the kernel adds them
+        total = total + shares.tensor[i]
+    delta = total.to(dtype)
+    w = 1.0 + 0.1 * rnd(H, seed=3)
+    for rows in (None, torch.tensor([R - 1, 0, R // 2], dtype=torch.int32, device=DEV)):
+        M = R if rows is None else 3
+        ha, hb = rnd(R, H, seed=1, scale=3.0), rnd(R, H, seed=1, scale=3.0)
+        a = torch.empty(M, H, dtype=dtype, device=DEV)
+        b = torch.empty_like(a)
+        ops.add_rmsnorm(ha, shares, w, 1e-5, a, rows)
+        ref.add_rmsnorm(hb, delta, w, 1e-5, b, rows)
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+        torch.testing.assert_close(ha, hb, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("M", [8, 17, 64])
+def test_product_for_the_residual_stream_in_every_form(ops, monkeypatch, M):
+    """linear_residual under every way the plan may name: bfloat16 rows or shares whose sum is the product."""
+    from return_amd.parts.runtime import Slabs
+    plan = {}
+    monkeypatch.setattr(ops, "product_plan", plan)
+    N, K = 520, 1024
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=M), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.2)
+    want = x.double() @ w.double().t()
+    ways = ops._candidates(M, N, K, False, "residual")
+    assert ("split4" in ways) == (M > 16) and "library" in ways
+    for how in ways:
+        plan.clear()
+        plan[(ops._rows_step(M), N, K, False, "residual")] = how
+        y = ops.linear_residual(x, w)
+        if how.startswith("split"):
+            assert isinstance(y, Slabs) and tuple(y.tensor.shape) == (int(how[5:]), M, N) and y.tensor.dtype == torch.float32
+            torch.testing.assert_close(y.tensor.double().sum(0), want, atol=1e-3, rtol=1e-4)
+        else:
+            torch.testing.assert_close(y.float(), want.float(), **tol(torch.bfloat16))
+    plan.clear()
+    # the rule: many columns of K against few of N, 17 to 64 rows
+    assert ops.route_linear(64, 4096, 12288, "residual") == "split4" and ops.route_linear(16, 4096, 12288, "residual") != "split4"
+    assert not ops.route_linear(64, 4096, 4096, "residual").startswith("split")
+
+
 def test_norms_are_not_deferred_where_the_sweep_does_not_form_the_products(ops):
     bf = torch.bfloat16
     w1, w2 = rnd(512, 264, dtype=bf), rnd(300, 512, dtype=bf)

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from return_amd.parts.runtime import ScaledRows
+from return_amd.parts.runtime import ScaledRows, Slabs
 
 
 class TorchOps:
@@ -23,6 +23,8 @@ class TorchOps:
 
     # rollout/fused.py:6-17 with the residual addition of qwen3.py:63,67 in front
     def add_rmsnorm(self, h, delta, weight, eps, out, rows=None):
+        if isinstance(delta, Slabs):                        # shares of a product: their sum, rounded as the product would be
+            delta = delta.tensor.sum(0).to(out.dtype)
         if rows is None:
             if delta is not None:
                 h += delta.float()
@@ -112,6 +114,14 @@ class TorchOps:
     @staticmethod
     def _rstd(rows):
         return 1.0 / torch.sqrt(rows.partials.sum(-1, keepdim=True) / rows.size + rows.eps)
+
+    def linear_residual(self, x, w):
+        """As HipOps: for more than 16 rows the product comes as two shares over halves of K."""
+        if isinstance(x, ScaledRows) or x.shape[0] <= 16 or x.shape[1] % 2:
+            return self.linear(x, w)
+        half = x.shape[1] // 2
+        return Slabs(torch.stack([x[:, :half].float() @ w[:, :half].float().t(),
+                                  x[:, half:].float() @ w[:, half:].float().t()]))
 
     def can_defer_norm(self, M, w_last, w_first, gated_first):
         return 1 <= M <= 16 and w_first.shape[1] == w_last.shape[0] >= self.SHARES
