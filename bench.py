@@ -235,7 +235,7 @@ def continuous_4b(args):
     from return_amd.engine import Engine
     n = args.batch if args.batch != 8 else 128
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_4B, use_graphs=not args.no_graphs,
-                               tune_products=not args.no_tune,
+                               tune_products=not args.no_tune, defer_norms=not args.no_defer_norms,
                                max_token=n * 4608, max_step_tokens=512 + n, prefill_chunk=512)
     eng = Engine(runner=runner)
     rnd = random.Random(0)
@@ -273,7 +273,7 @@ def long_32b(args):
     elt = 2 if args.dtype == "bfloat16" else 4
     n, ctx, new, long_ctx = 16, 8192, max(2, args.steps), 32768
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_32B, std=0.01, use_graphs=not args.no_graphs,
-                               tune_products=not args.no_tune,
+                               tune_products=not args.no_tune, defer_norms=not args.no_defer_norms,
                                max_token=n * (ctx + 512) + long_ctx, max_step_tokens=ctx, prefill_chunk=ctx)
     eng = Engine(runner=runner)
     rnd = random.Random(1)

@@ -60,6 +60,8 @@ class ModelRunner:
         del weights
         if ec.tune_products and self.rt.dtype == torch.bfloat16 and hasattr(self.rt.ops, "tune_products"):
             self.rt.ops.tune_products(self.rt.products, max_rows=ec.max_reside)
+            if ec.defer_norms and hasattr(self.rt.ops, "tune_norm_pairs"):
+                self.rt.ops.tune_norm_pairs(self.rt.norm_pairs, max_rows=ec.max_reside)
         self._check_cache_fits()
         self.cache = CacheManager(self.model.cache_layers(), ec.page_size, ec.max_token,
                                   ec.max_reside, self.rt.dtype, self.rt.device)

@@ -93,6 +93,8 @@ def _ptr(t: Optional[torch.Tensor]):
 # What tune_products has measured in this process: (row step, N, K, gated, result dtype) -> the way that
 # beat the rule's, or None where the rule stands. Every kernel set that tunes gets the same answers.
 _PRODUCTS_MEASURED = {}
+_PRODUCT_TIMES = {}        # the same keys -> {way: seconds}, as measured
+_NORM_PAIRS_MEASURED = {}  # (row step, shape of the product before a norm, of the one after, gated) -> the norm inside them is faster
 
 
 class HipOps:
@@ -136,6 +138,8 @@ class HipOps:
                                          <= 2e-5 * want.abs().max()).item())
         self.product_plan = {}               # (row step, N, K, gated, result dtype) -> way, where measured faster than the rule
         self._measured = _PRODUCTS_MEASURED
+        self._times = _PRODUCT_TIMES
+        self._defer = {}                     # as _NORM_PAIRS_MEASURED, for the pairs this kernel set has been shown
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -439,7 +443,55 @@ class HipOps:
             return False
         if self.lib.ra_gemm_sweep_workgroups(H, self.cu_count) > 256:      # shares of a row's sum that the next product adds up
             return False
-        return bool(self.lib.ra_gemm_sweep_fits(M, w_last.shape[1]) and self.lib.ra_gemm_sweep_fits(M, H))
+        if not (self.lib.ra_gemm_sweep_fits(M, w_last.shape[1]) and self.lib.ra_gemm_sweep_fits(M, H)):
+            return False
+        # measured at load (tune_norm_pairs) where it was; else yes
+        hit = self._defer.get((self._rows_step(M), tuple(w_last.shape), tuple(w_first.shape), bool(gated_first)))
+        return True if hit is None else hit
+
+    def tune_norm_pairs(self, pairs, max_rows=16):
+        """Measures, for every shape among ``pairs`` and every row count of ROW_STEPS up to 16, whether the
+        norm between two products is faster finished inside them (which ties both to the sweep) or as a
+        kernel of its own between the fastest ways to form them, and notes it for can_defer_norm.
+        pairs: (w_last [H, K1], norm weight [H] fp32, eps, w_first, gated) as the model has them."""
+        groups = {}
+        for w_last, wn, eps, w_first, gated in pairs:
+            if w_last.dtype != torch.bfloat16 or w_first.dtype != torch.bfloat16 or w_last.device != self.device:
+                continue
+            groups.setdefault((tuple(w_last.shape), tuple(w_first.shape), bool(gated)), []).append((w_last, wn, eps, w_first))
+        for (s_last, s_first, gated), members in groups.items():
+            for rows in self.ROW_STEPS:
+                if rows > 16 or (rows > max(1, max_rows) and rows != self._rows_step(max_rows)):
+                    continue
+                key = (rows, s_last, s_first, gated)
+                if key in _NORM_PAIRS_MEASURED:
+                    self._defer[key] = _NORM_PAIRS_MEASURED[key]
+                    continue
+                self._defer.pop(key, None)
+                if not self.can_defer_norm(rows, members[0][0], members[0][3], gated):
+                    continue
+                _NORM_PAIRS_MEASURED[key] = self._defer[key] = self._measure_norm_pair(rows, members[:16], gated)
+
+    def _measure_norm_pair(self, rows, members, gated):
+        H, K1 = members[0][0].shape
+        x = torch.randn(rows, K1, device=self.device, dtype=torch.float32).to(torch.bfloat16)
+        h = torch.randn(rows, H, device=self.device, dtype=torch.float32)
+        out = torch.empty(rows, H, dtype=torch.bfloat16, device=self.device)
+        finish = self.linear_silu_mul if gated else self.linear
+
+        def inside(m):
+            w_last, wn, eps, w_first = m
+            return finish(self.linear_add_norm(x, w_last, h, wn, eps), w_first)
+
+        def apart(m):
+            w_last, wn, eps, w_first = m
+            self.add_rmsnorm(h, self.linear_residual(x, w_last), wn, eps, out)
+            return finish(out, w_first)
+        launches = max(4, min(16, len(members)))
+        t_in = self._time_over(inside, members, launches)
+        h.normal_()
+        t_out = self._time_over(apart, members, launches)
+        return t_in <= t_out
 
     def _sweep_norm(self, x, w, gated, out_dtype, rows_in=None, h=None, w_next=None):
         """The sweeping product with a row scale from rows_in (ScaledRows) and, with h, the residual epilogue."""
@@ -641,6 +693,7 @@ class HipOps:
                     times[how] += int(how[5:]) * rows * N * 4 / 1.5e12
         finally:
             self.product_plan = saved
+        self._times[key] = dict(times)
         best = min(times, key=times.get)
         return best if best != rule and times[best] < margin * times[rule] else None
 

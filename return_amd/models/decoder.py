@@ -42,6 +42,16 @@ class Decoder:
         for call in self.schedule:
             if not 0 <= call.block < len(self.blocks):
                 raise ValueError(f"run order names block {call.block}, the model has {len(self.blocks)}")
+        # the norms that sit between two products (inside a block, and between one block and the next in
+        # the run order), for the kernel set to measure whether it finishes them inside those products
+        for i, call in enumerate(self.schedule):
+            block = self.blocks[call.block]
+            rt.norm_pairs.extend(block.norm_pairs() if hasattr(block, "norm_pairs") else [])
+            nxt = self.blocks[self.schedule[i + 1].block] if i + 1 < len(self.schedule) else None
+            last = getattr(block, "last_product", None)
+            if nxt is not None and last is not None and getattr(nxt, "first_product", None) is not None and \
+                    hasattr(getattr(nxt, "first_norm", None), "weight"):
+                rt.norm_pairs.append((last, nxt.first_norm.weight, nxt.first_norm.eps, *nxt.first_product))
         rt.forget_casts()
 
     def cache_layers(self):

@@ -49,6 +49,15 @@ class PreNormBlock:
         # what the block before may fuse into: this block's first norm and the product behind it
         self.first_norm = self.mixer_norm
         self.first_product = getattr(self.mixer, "first_product", None)
+        self.last_product = getattr(self.feed_forward, "last_product", None)
+
+    def norm_pairs(self):
+        """(product before, norm weight, eps, product after, gated) of the norm inside the block, if it sits
+        between two products."""
+        last, first = getattr(self.mixer, "last_product", None), getattr(self.feed_forward, "first_product", None)
+        if last is None or first is None or not hasattr(self.feed_forward_norm, "weight"):
+            return []
+        return [(last, self.feed_forward_norm.weight, self.feed_forward_norm.eps, *first)]
 
     def cache_spec(self):
         return self.mixer.cache_spec()

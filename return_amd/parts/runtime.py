@@ -94,6 +94,7 @@ class Runtime:
         self.ops = ops
         self._cast: Dict[int, torch.Tensor] = {}
         self.products = []                  # (weight, gated, result dtype) of the parts' matrix products
+        self.norm_pairs = []                # (weight before, norm weight, eps, weight after, gated) of norms between two products
 
     # ---- weight preparation -------------------------------------------------
     def matrix(self, t: torch.Tensor) -> torch.Tensor:

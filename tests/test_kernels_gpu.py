@@ -386,7 +386,7 @@ def test_product_for_the_residual_stream_in_every_form(ops, monkeypatch, M):
     assert not ops.route_linear(64, 4096, 4096, "residual").startswith("split")
 
 
-def test_norms_are_not_deferred_where_the_sweep_does_not_form_the_products(ops):
+def test_norms_are_not_deferred_where_the_sweep_does_not_form_the_products(ops, monkeypatch):
     bf = torch.bfloat16
     w1, w2 = rnd(512, 264, dtype=bf), rnd(300, 512, dtype=bf)
     assert ops.can_defer_norm(16, w1, w2, False)
@@ -395,6 +395,29 @@ def test_norms_are_not_deferred_where_the_sweep_does_not_form_the_products(ops):
     assert not ops.can_defer_norm(4, w1.float(), w2.float(), False)     # float32: the plain kernels
     assert not ops.can_defer_norm(4, rnd(100, 264, dtype=bf), rnd(300, 100, dtype=bf), False)   # narrower than the chip
     assert not ops.can_defer_norm(4, w1, rnd(300, 520, dtype=bf), False)   # widths that do not meet
+    # where a pair has been measured at load, the measurement decides
+    monkeypatch.setattr(ops, "_defer", {(4, (512, 264), (300, 512), False): False})
+    assert not ops.can_defer_norm(4, w1, w2, False) and ops.can_defer_norm(16, w1, w2, False)
+
+
+def test_norm_pairs_are_measured_at_load(ops, monkeypatch):
+    """tune_norm_pairs times every pair of products with a norm between them both ways, at the row counts
+    up to 16, once in a process, and can_defer_norm follows what it found."""
+    import return_amd.kernels.hip_ops as ho
+    monkeypatch.setattr(ops, "_defer", {})
+    monkeypatch.setattr(ho, "_NORM_PAIRS_MEASURED", {})
+    bf = torch.bfloat16
+    pairs = [(rnd(512, 264, dtype=bf, seed=i), 1.0 + 0.1 * rnd(512, seed=9), 1e-5, rnd(600, 512, dtype=bf, seed=20 + i), True)
+             for i in range(3)]
+    ops.tune_norm_pairs(pairs, max_rows=5)
+    assert set(ops._defer) == {(r, (512, 264), (600, 512), True) for r in (1, 2, 4, 8)}
+    assert all(isinstance(v, bool) for v in ops._defer.values())
+    for (r, _, _, _), v in ops._defer.items():
+        assert ops.can_defer_norm(r, pairs[0][0], pairs[0][3], True) == v
+    calls = []
+    monkeypatch.setattr(ops, "_time_over", lambda *a: calls.append(a) or 1.0)
+    ops.tune_norm_pairs(pairs, max_rows=5)
+    assert not calls                                                       # nothing is measured twice
 
 
 def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
