@@ -404,6 +404,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel from the host instead of replaying HIP graphs")
+    ap.add_argument("--page-size", type=int, default=PAGE, help=f"tokens per cache page (the benchmark's is {PAGE})")
     ap.add_argument("--no-defer-norms", action="store_true",
                     help="run every RMSNorm as a kernel of its own instead of inside the products around it")
     ap.add_argument("--no-tune", action="store_true",
@@ -425,7 +426,7 @@ def main():
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),
                                use_graphs=not args.no_graphs, tune_products=not args.no_tune,
-                               defer_norms=not args.no_defer_norms)
+                               defer_norms=not args.no_defer_norms, page_size=args.page_size)
     V = cfg.vocab_size
 
     def roofline(batch, ms, new_before, steps):
@@ -501,7 +502,7 @@ def main():
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": cfg.intermediate_size, "vocab": V, "global_batch": args.batch,
-                   "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": PAGE,
+                   "seq_len": CONTEXT, "max_context": MAX_CONTEXT, "page_size": args.page_size,
                    "new_tokens": args.warmup + args.steps, "parallelism": "single GPU",
                    "hip_graphs": not args.no_graphs, "tuned_products": not args.no_tune,
                    "norms_in_products": not args.no_defer_norms, "weights": "random N(0,0.02)"},

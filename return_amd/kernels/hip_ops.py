@@ -787,14 +787,15 @@ class HipOps:
         request's splits are the waves of one workgroup that merges them itself (no partial sums
         in memory, no merge kernel). Measured on MI355X: that is 3 to 11 % faster when the
         (request, kv head) pairs are a whole number of rounds over the CUs (batch 32, 64, 96, 128 with
-        8 kv heads) and slower otherwise: a workgroup of eight waves fills a CU's LDS, and its waves
-        walk through their passes one after the other."""
+        8 kv heads) or at least three rounds (batch 100 of uneven lengths: 208 against 221 µs), and
+        slower otherwise (batch 40, 48, 72: 5 to 15 %): a workgroup of eight waves fills a CU's LDS, and
+        a last round that is far from full leaves most of the chip idle."""
         longest = step.max_decode_seq_len
         S = self.decode_split_tokens
         groups = step.n_decode * n_kv * -(-(n_q // n_kv) // 16)
         waves = self.lib.ra_attention_decode_merge_waves(D)
         if S <= 0 and window == 0 and waves >= 2 and longest > 64 and self.decode_merge_round > 0 \
-                and groups % self.decode_merge_round == 0:
+                and (groups % self.decode_merge_round == 0 or groups >= 3 * self.decode_merge_round):
             # (the kernel cuts every request into W even splits of its own length)
             W = min(waves, -(-longest // 64))
             return 64, W, True
