@@ -616,13 +616,14 @@ def test_prefill_attention_every_head_size(ops, ref, D, key_split, monkeypatch):
         torch.testing.assert_close(a.float(), b.float(), **tol(torch.bfloat16))
 
 
-@pytest.mark.parametrize("merge", [False, True])
+@pytest.mark.parametrize("merge", [0, 2, 4, 8])
 @pytest.mark.parametrize("D", list(range(16, 257, 16)))
 def test_decode_attention_every_head_size(ops, ref, monkeypatch, D, merge):
     """The bfloat16 decode kernel at every head size it takes, grouped, ungrouped and with more
     query heads to a kv head than one wave takes; with the splits of a request merged by a
-    second kernel, and as the waves of one workgroup that merges them itself."""
+    second kernel, and as two, four or eight waves of one workgroup that merges them itself."""
     monkeypatch.setattr(ops, "decode_merge_round", 1 if merge else 0)
+    monkeypatch.setattr(ops, "decode_merge_waves", merge)
     for Hq, Hkv in ((4, 1), (3, 3), (16, 2), (34, 2)):
         P = 16
         segs = [(1, 150), (1, 1), (1, 64), (1, 700)]
@@ -639,7 +640,8 @@ def test_decode_attention_every_head_size(ops, ref, monkeypatch, D, merge):
         ops.attention(q, a, kp, vp, step, 0, D ** -0.5, 0)
         ref.attention(q, b, kp, vp, step, 0, D ** -0.5, 0)
         torch.testing.assert_close(a.float(), b.float(), **tol(torch.bfloat16))
-        assert ops._decode_splits(step, Hq, Hkv, D, 0)[2] == merge
+        S, W, merged = ops._decode_splits(step, Hq, Hkv, D, 0)
+        assert merged == bool(merge) and (not merge or W == min(merge, ops.lib.ra_attention_decode_merge_waves(D)))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -699,7 +701,7 @@ def test_attention_far_key_stands_out(ops, dtype):
     torch.testing.assert_close(out[0, ::2].float(), want, atol=3e-2, rtol=3e-2)
 
 
-@pytest.mark.parametrize("split", [0, 64, 192, "merge"])
+@pytest.mark.parametrize("split", [0, 64, 192, "merge", "merge8"])
 @pytest.mark.parametrize("D,Hq,Hkv,normed,rotated,window", [
     (128, 8, 2, True, True, 0), (64, 4, 4, True, True, 0), (192, 3, 1, False, True, 0), (256, 4, 2, True, False, 0),
     (128, 40, 2, True, True, 0), (64, 6, 2, True, True, 70), (128, 4, 1, False, False, 0)])
@@ -707,8 +709,10 @@ def test_decode_attention_that_prepares_q_k_v_itself(ops, monkeypatch, D, Hq, Hk
     """The decode kernel fed with the projection's output (it norms and rotates q and k and writes
     k and v into the cache) against the preparation kernel followed by the decode kernel: new
     tokens at the first place, at the edges of pages, passes and splits, and far out."""
-    monkeypatch.setattr(ops, "decode_split_tokens", 0 if split == "merge" else split)
-    monkeypatch.setattr(ops, "decode_merge_round", 1 if split == "merge" else 0)
+    merge = str(split).startswith("merge")
+    monkeypatch.setattr(ops, "decode_split_tokens", 0 if merge else split)
+    monkeypatch.setattr(ops, "decode_merge_round", 1 if merge else 0)
+    monkeypatch.setattr(ops, "decode_merge_waves", 8 if split == "merge8" else 0)
     P = 16
     starts = [0, 1, 15, 16, 63, 64, 65, 127, 128, 191, 192, 700]
     need = [-(-(a + 1) // P) for a in starts]
