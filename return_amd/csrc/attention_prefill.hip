@@ -379,21 +379,23 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
 #define PRE_CAT2(a, b) a##b
 #define PRE_CAT(a, b) PRE_CAT2(a, b)
 // head sizes 16*(4*PRE_PART+1) .. 16*(4*PRE_PART+4)
-extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out,
+extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, int tile_rows, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out,
                                               const bf16* kp, const bf16* vp, const int* pt,
                                               const int* cup, const int* kvs, const int* cuq,
                                               const int* qs, const int* tiles, int n_tiles, int Hq,
                                               int Hkv, int P, float scale, int window) {
+#define PRE_LAUNCH(N, QG_, KS_)                                                                    \
+    hipLaunchKernelGGL((attn_prefill_kernel<N, QG_, KS_>), grid, dim3(256 * KS_), 0, st, q, out, kp, vp, pt, \
+                       cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window)
 #define PRE_CASE(N)                                                                               \
     case N:                                                                                       \
-        if (key_split == 2 && N <= PRE_WIDE_D16)                                                      \
-            hipLaunchKernelGGL((attn_prefill_kernel<N, (N <= PRE_WIDE_D16 ? 2 : 1), (N <= PRE_WIDE_D16 ? 2 : 1)>), \
-                               grid, dim3(512), 0, st, q, out, kp, vp, pt, cup, kvs, cuq, qs, tiles,      \
-                               n_tiles, Hq, Hkv, P, scale, window);                                       \
-        else                                                                                          \
-            hipLaunchKernelGGL((attn_prefill_kernel<N, (N <= PRE_WIDE_D16 ? 2 : 1), 1>), grid, dim3(256), \
-                               0, st, q, out, kp, vp, pt, cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P,  \
-                               scale, window);                                                        \
+        if (N <= PRE_WIDE_D16 && tile_rows == 128) {                                              \
+            if (key_split == 2) PRE_LAUNCH(N, (N <= PRE_WIDE_D16 ? 2 : 1), (N <= PRE_WIDE_D16 ? 2 : 1)); \
+            else PRE_LAUNCH(N, (N <= PRE_WIDE_D16 ? 2 : 1), 1);                                   \
+        } else {                                                                                  \
+            if (key_split == 2 && N <= PRE_WIDE_D16) PRE_LAUNCH(N, 1, (N <= PRE_WIDE_D16 ? 2 : 1)); \
+            else PRE_LAUNCH(N, 1, 1);                                                             \
+        }                                                                                         \
         return RA_OK;
     switch (D16) {
         PRE_CASE(4 * PRE_PART + 1) PRE_CASE(4 * PRE_PART + 2) PRE_CASE(4 * PRE_PART + 3)
@@ -401,11 +403,12 @@ extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, int key_split, dim3 grid
         default: return RA_ERR_ARG;
     }
 #undef PRE_CASE
+#undef PRE_LAUNCH
 }
 #endif  // PRE_PART
 
 #ifdef PRE_API
-#define PRE_PART_ARGS int D16, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
+#define PRE_PART_ARGS int D16, int tile_rows, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
     const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs,    \
     const int* tiles, int n_tiles, int Hq, int Hkv, int P, float scale, int window
 extern "C" int ra_pre_part_0(PRE_PART_ARGS);
@@ -413,7 +416,8 @@ extern "C" int ra_pre_part_1(PRE_PART_ARGS);
 extern "C" int ra_pre_part_2(PRE_PART_ARGS);
 extern "C" int ra_pre_part_3(PRE_PART_ARGS);
 
-// Rows of a q tile for head size D: 128 up to head size 128, 64 beyond.
+// Rows of a q tile for head size D: 128 up to head size 128, 64 beyond. Up to head size 128 tiles of 64
+// rows are taken too (one group of rows per wave: more LDS traffic per flop, twice the workgroups).
 extern "C" int ra_attention_prefill_tile_rows(int D) { return D <= 16 * PRE_WIDE_D16 ? 128 : 64; }
 
 // tiles: int32 [n_tiles][2] = (request number, first row of the tile within the request's new
@@ -427,7 +431,7 @@ extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k
                                          float scale, int window, void* stream) {
     if (n_tiles <= 0) return RA_OK;
     if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 ||
-        (long long)n_tiles * Hq > 0x7fffffffLL || tile_rows != ra_attention_prefill_tile_rows(D))
+        (long long)n_tiles * Hq > 0x7fffffffLL || (tile_rows != ra_attention_prefill_tile_rows(D) && tile_rows != 64))
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(n_tiles * Hq);
@@ -439,7 +443,7 @@ extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k
     if (key_split > 2) return RA_ERR_ARG;
     int rc;
 #define GO(k)                                                                                      \
-    rc = ra_pre_part_##k(d16, key_split, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
+    rc = ra_pre_part_##k(d16, tile_rows, key_split, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tiles, \
                          n_tiles, Hq, Hkv, P, scale, window)
     switch ((d16 - 1) / 4) {

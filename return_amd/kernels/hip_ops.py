@@ -115,6 +115,7 @@ class HipOps:
         self.decode_merge_round = self.cu_count
         self.decode_merge_waves = 0          # waves of such a workgroup; 0: by the number of pairs and the context
         self.prefill_key_split = 0           # groups of waves that share a q tile's keys (1 or 2); 0: by the number of tiles
+        self.prefill_small_tiles = True      # q tiles of 64 rows instead of 128 while those would not fill the chip
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
         self.own_gemm = False                # True: bf16 products of many rows use the hand-written MFMA kernel
@@ -729,10 +730,12 @@ class HipOps:
         _code(dtype)
 
     def prefill_tile_rows(self, D, dtype):
-        """Rows per q tile of the list that attention() reads from step.prefill_tiles for requests with
-        more than one token, or None where the kernel that serves this head size takes no list."""
+        """Rows per q tile of the lists that attention() reads from step.prefill_tiles for requests with
+        more than one token (a tuple; the first is the one it needs, the others it uses when they are
+        there), or None where the kernel that serves this head size takes no list."""
         if dtype == torch.bfloat16 and D % 16 == 0 and D <= 256:
-            return int(self.lib.ra_attention_prefill_tile_rows(D))
+            rows = int(self.lib.ra_attention_prefill_tile_rows(D))
+            return (rows,) if rows == 64 else (rows, 64)
         return None
 
     def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
@@ -773,7 +776,16 @@ class HipOps:
             tiles = step.prefill_tiles.get(rows)
             if tiles is None:
                 raise KernelError(f"attention: the step lists no q tiles of {rows} rows (head size {D})")
-            split = self.prefill_key_split or self._prefill_key_split(step, rows, tiles.shape[0] * n_q)
+            # Few tiles (a portion of 512 rows is four or five of 128 rows: 128 to 160 workgroups with 32
+            # heads) leave CUs idle: tiles of 64 rows, one group of rows per wave and two groups of waves a
+            # tile, make twice the workgroups of less than half the work each (measured at 32 heads of 128:
+            # 512 rows over 4,096 keys 78 µs against 109, 300 rows at 1,500 beside 212 from scratch 36
+            # against 50; from 1,024 rows on slower)
+            small = step.prefill_tiles.get(64) if rows == 128 else None
+            small_split = 0
+            if small is not None and self.prefill_small_tiles and 2 * small.shape[0] * n_q <= 3 * self.cu_count:
+                rows, tiles, small_split = 64, small, 2
+            split = self.prefill_key_split or small_split or self._prefill_key_split(step, rows, tiles.shape[0] * n_q)
             self._check(self.lib.ra_attention_prefill_bf16(
                 _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], rows,
                 split, n_q, n_kv, D, P, float(scale), window, self._stream()),

@@ -70,7 +70,7 @@ class PagedAttention:
         """The q-tile list that the kernel set's attention reads for requests with more than one token."""
         ops = self.rt.ops
         rows = ops.prefill_tile_rows(self.d, self.rt.dtype) if hasattr(ops, "prefill_tile_rows") else None
-        return {"prefill_tile_rows": {rows}} if rows else {}
+        return {"prefill_tile_rows": set(rows)} if rows else {}
 
     def forward(self, x, step, cache, write_cache=True, sink=None):
         rt, ops = self.rt, self.rt.ops

@@ -571,7 +571,8 @@ ATTN_CASES = [
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,D,P,segs,window", ATTN_CASES)
-def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
+def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window, monkeypatch):
+    monkeypatch.setattr(ops, "prefill_small_tiles", (Hq + D + len(segs)) % 2 == 0)     # tiles of 64 rows in half the cases
     q_lens = [s[0] for s in segs]
     q_starts = [s[1] for s in segs]
     need = [-(-(a + b) // P) for a, b in segs]
@@ -591,13 +592,18 @@ def test_attention(ops, ref, dtype, Hq, Hkv, D, P, segs, window):
     torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("small_tiles", [False, True])
 @pytest.mark.parametrize("key_split", [1, 2])
 @pytest.mark.parametrize("D", list(range(16, 257, 16)))
-def test_prefill_attention_every_head_size(ops, ref, D, key_split, monkeypatch):
+def test_prefill_attention_every_head_size(ops, ref, D, key_split, small_tiles, monkeypatch):
     """The bfloat16 prefill kernel at every head size it takes: whole prompts, portions with
     context, tiles that end inside a page, a window, an odd and an even number of key tiles;
-    with one group of waves per q tile and with two that share its keys."""
+    with one group of waves per q tile and with two that share its keys; with q tiles of 128 rows
+    and (up to head size 128, while they are few) of 64."""
+    if small_tiles and D > 128:
+        pytest.skip("beyond head size 128 the tiles have 64 rows anyway")
     monkeypatch.setattr(ops, "prefill_key_split", key_split)
+    monkeypatch.setattr(ops, "prefill_small_tiles", small_tiles)
     for (Hq, Hkv), window in (((4, 2), 0), ((3, 1), 37)):
         P = 16
         segs = [(70, 0), (2, 131), (65, 64), (5, 3), (130, 259), (140, 300)]
