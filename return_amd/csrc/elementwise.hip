@@ -180,33 +180,47 @@ __global__ void add_slabs_rmsnorm_kernel(float* __restrict__ h, const float* __r
     }
 }
 
-// The same for H % 4 == 0, H <= 4096 and S shares known at compile time: 16-byte accesses, every load of
-// a thread asked for at once, the row kept in registers between the two phases. 1024 threads a row.
-template <typename T, int S>
+// The same for H % 4 == 0, H <= 4096 C4 and S shares known at compile time: 16-byte accesses, every load
+// of a thread asked for at once, the row kept in registers between the two phases. 1024 threads a row,
+// C4 pieces of four columns a thread (piece i of thread c: columns 4 (c + 1024 i) ..).
+template <typename T, int S, int C4>
 __global__ __launch_bounds__(1024) void add_slabs_rmsnorm_vec_kernel(
     float* __restrict__ h, const float* __restrict__ slabs, size_t slab_stride, const float* __restrict__ w, float eps,
     T* __restrict__ out, const int* __restrict__ rows, int H) {
     __shared__ float scratch[16];
-    const int m = blockIdx.x, c = threadIdx.x;
+    const int m = blockIdx.x;
     const size_t r = rows ? (size_t)rows[m] : (size_t)m;
-    const bool in = c < (H >> 2);
-    const int cc = in ? c : 0;
-    float4 v = reinterpret_cast<const float4*>(h + r * H)[cc];
-    float4 sh[S];
+    bool in[C4];
+    int cc[C4];
+    float4 v[C4], ww[C4], sh[C4][S];
 #pragma unroll
-    for (int s = 0; s < S; ++s) sh[s] = reinterpret_cast<const float4*>(slabs + (size_t)s * slab_stride + r * H)[cc];
-    const float4 ww = reinterpret_cast<const float4*>(w)[cc];
-    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = 0; i < C4; ++i) {
+        const int c = threadIdx.x + 1024 * i;
+        in[i] = c < (H >> 2);
+        cc[i] = in[i] ? c : 0;
+        v[i] = reinterpret_cast<const float4*>(h + r * H)[cc[i]];
 #pragma unroll
-    for (int s = 0; s < S; ++s) { d.x += sh[s].x; d.y += sh[s].y; d.z += sh[s].z; d.w += sh[s].w; }
-    v.x += round_to<T>(d.x); v.y += round_to<T>(d.y); v.z += round_to<T>(d.z); v.w += round_to<T>(d.w);
-    if (in && rows == nullptr) reinterpret_cast<float4*>(h + r * H)[c] = v;
-    float ss = in ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f;
+        for (int s = 0; s < S; ++s) sh[i][s] = reinterpret_cast<const float4*>(slabs + (size_t)s * slab_stride + r * H)[cc[i]];
+        ww[i] = reinterpret_cast<const float4*>(w)[cc[i]];
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < C4; ++i) {
+        float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int s = 0; s < S; ++s) { d.x += sh[i][s].x; d.y += sh[i][s].y; d.z += sh[i][s].z; d.w += sh[i][s].w; }
+        v[i].x += round_to<T>(d.x); v[i].y += round_to<T>(d.y); v[i].z += round_to<T>(d.z); v[i].w += round_to<T>(d.w);
+        if (in[i] && rows == nullptr) reinterpret_cast<float4*>(h + r * H)[cc[i]] = v[i];
+        ss += in[i] ? v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w : 0.f;
+    }
     ss = block_sum(ss, scratch);
     const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
-    if (in) {
-        T* o = out + (size_t)m * H + 4 * c;
-        const float a = v.x * rstd * ww.x, b = v.y * rstd * ww.y, e = v.z * rstd * ww.z, f = v.w * rstd * ww.w;
+#pragma unroll
+    for (int i = 0; i < C4; ++i) {
+        if (!in[i]) continue;
+        T* o = out + (size_t)m * H + 4 * cc[i];
+        const float a = v[i].x * rstd * ww[i].x, b = v[i].y * rstd * ww[i].y, e = v[i].z * rstd * ww[i].z,
+                    f = v[i].w * rstd * ww[i].w;
         if constexpr (sizeof(T) == 2) {
             uint2 p;
             p.x = (uint32_t)f2bf_bits(a) | ((uint32_t)f2bf_bits(b) << 16);
@@ -218,13 +232,13 @@ __global__ __launch_bounds__(1024) void add_slabs_rmsnorm_vec_kernel(
     }
 }
 
-template <typename T>
+template <typename T, int C4>
 static bool launch_slabs_vec(int n_slabs, dim3 grid, hipStream_t st, float* h, const float* slabs, size_t stride,
                              const float* w, float eps, T* out, const int* rows, int H) {
     switch (n_slabs) {
-        case 2: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 2>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
-        case 4: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 4>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
-        case 8: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 8>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
+        case 2: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 2, C4>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
+        case 4: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 4, C4>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
+        case 8: hipLaunchKernelGGL((add_slabs_rmsnorm_vec_kernel<T, 8, C4>), grid, dim3(1024), 0, st, h, slabs, stride, w, eps, out, rows, H); return true;
         default: return false;
     }
 }
@@ -239,8 +253,13 @@ extern "C" int ra_add_slabs_rmsnorm(float* h, const float* slabs, int n_slabs, l
     dim3 grid(M);
     if (H % 4 == 0 && H <= 4096) {
         const bool done = dtype == RA_DTYPE_F32
-            ? launch_slabs_vec<float>(n_slabs, grid, st, h, slabs, stride, w, eps, (float*)out, rows, H)
-            : launch_slabs_vec<bf16>(n_slabs, grid, st, h, slabs, stride, w, eps, (bf16*)out, rows, H);
+            ? launch_slabs_vec<float, 1>(n_slabs, grid, st, h, slabs, stride, w, eps, (float*)out, rows, H)
+            : launch_slabs_vec<bf16, 1>(n_slabs, grid, st, h, slabs, stride, w, eps, (bf16*)out, rows, H);
+        if (done) return ra_launch_status();
+    } else if (H % 4 == 0 && H <= 8192) {
+        const bool done = dtype == RA_DTYPE_F32
+            ? launch_slabs_vec<float, 2>(n_slabs, grid, st, h, slabs, stride, w, eps, (float*)out, rows, H)
+            : launch_slabs_vec<bf16, 2>(n_slabs, grid, st, h, slabs, stride, w, eps, (bf16*)out, rows, H);
         if (done) return ra_launch_status();
     }
     dim3 block(H >= 2048 ? 1024 : 256);

@@ -59,7 +59,8 @@ class ModelRunner:
         self.model = Decoder(self.spec, weights, self.rt)
         del weights
         if ec.tune_products and self.rt.dtype == torch.bfloat16 and hasattr(self.rt.ops, "tune_products"):
-            self.rt.ops.tune_products(self.rt.products, max_rows=ec.max_reside)
+            self.rt.ops.tune_products(self.rt.products, max_rows=ec.max_reside,
+                                      max_rows_residual=ec.max_reside + min(ec.max_step_tokens, ec.prefill_chunk))
             if ec.defer_norms and hasattr(self.rt.ops, "tune_norm_pairs"):
                 self.rt.ops.tune_norm_pairs(self.rt.norm_pairs, max_rows=ec.max_reside)
         self._check_cache_fits()

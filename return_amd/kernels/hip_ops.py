@@ -360,9 +360,14 @@ class HipOps:
     # rule captures (the library streams one weight at 5.6 TB/s and the next at 2): route_* give the
     # rule's choice, tune_products replaces it where a measurement at load time says otherwise.
     ROW_STEPS = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64)     # row counts at which products are measured
+    # ... and beyond them the products for the residual stream only: with a few hundred rows (portions of
+    # prompts beside decoded tokens) the library gives a product with few result columns and many of K too
+    # few workgroups, and a batch over pieces of K is up to twice as fast (measured on MI355X, 512 rows:
+    # 8B down 84 -> 55 µs, 32B down 272 -> 122 µs)
+    ROW_STEPS_RESIDUAL = (96, 128, 192, 256, 384, 512, 640, 768, 1024)
 
-    def _rows_step(self, M):
-        for r in self.ROW_STEPS:
+    def _rows_step(self, M, residual=False):
+        for r in self.ROW_STEPS + (self.ROW_STEPS_RESIDUAL if residual else ()):
             if M <= r:
                 return r
         return 0                                          # more rows than are ever measured: the library
@@ -373,7 +378,7 @@ class HipOps:
         """How linear() forms a bfloat16 product of M rows: the measured choice if there is one, else the rule.
         out_dtype "residual": the product whose result goes into the residual stream (linear_residual), bfloat16
         rows or, "split<n>", n shares of 32-bit sums from the library's batched product over n pieces of K."""
-        hit = self.product_plan.get((self._rows_step(M), N, K, False, out_dtype))
+        hit = self.product_plan.get((self._rows_step(M, out_dtype == "residual"), N, K, False, out_dtype))
         if hit is not None:
             return hit
         if out_dtype == "residual":
@@ -640,7 +645,7 @@ class HipOps:
             c += [f"split{n}" for n in self.SPLITS if K % (8 * n) == 0]
         return c
 
-    def tune_products(self, products, max_rows=64, margin=0.93):
+    def tune_products(self, products, max_rows=64, margin=0.93, max_rows_residual=0):
         """Measures, for every shape among ``products`` and every row count of ROW_STEPS up to max_rows,
         the ways to form the product, and notes the fastest in product_plan where it beats the rule's
         choice by more than the margin (so that noise does not move a choice to and fro).
@@ -661,8 +666,12 @@ class HipOps:
                     seen.add(w.data_ptr())
                     uniq.append(w)
             launches = max(4, min(16, len(uniq)))
-            for rows in self.ROW_STEPS:
-                if rows > max(1, max_rows) and rows != self._rows_step(max_rows):
+            steps = self.ROW_STEPS
+            if out_dtype == "residual" and max_rows_residual > self.ROW_STEPS[-1]:
+                top = self._rows_step(max_rows_residual, True) or self.ROW_STEPS_RESIDUAL[-1]
+                steps = steps + tuple(r for r in self.ROW_STEPS_RESIDUAL if r <= top)
+            for rows in steps:
+                if rows <= self.ROW_STEPS[-1] and rows > max(1, max_rows) and rows != self._rows_step(max_rows):
                     continue
                 key = (rows, N, K, gated, out_dtype)
                 if key not in self._measured:
@@ -680,19 +689,22 @@ class HipOps:
             if len(cands) < 2 or rule not in cands:
                 return None
             x = torch.randn(rows, K, device=self.device, dtype=torch.float32).to(torch.bfloat16)
+            if out_dtype == "residual":
+                # with the residual add and norm that takes the result: shares cost it more than one result does
+                h = torch.zeros(rows, N, device=self.device, dtype=torch.float32)
+                wn = torch.ones(N, device=self.device, dtype=torch.float32)
+                normed = torch.empty(rows, N, device=self.device, dtype=torch.bfloat16)
             times = {}
             for how in cands:
                 if gated:
                     run = lambda w, how=how: self._gated_by(how, x, w)
                 elif how.startswith("split"):
-                    run = lambda w, how=how: self._split_product(x, w, int(how[5:]))
+                    run = lambda w, how=how: self.add_rmsnorm(h, self._split_product(x, w, int(how[5:])), wn, 1e-6, normed)
+                elif out_dtype == "residual":
+                    run = lambda w, how=how: self.add_rmsnorm(h, self._linear_by(how, x, w, torch.bfloat16), wn, 1e-6, normed)
                 else:
-                    run = lambda w, how=how: self._linear_by(how, x, w, torch.bfloat16 if out_dtype == "residual" else out_dtype)
+                    run = lambda w, how=how: self._linear_by(how, x, w, out_dtype)
                 times[how] = self._time_over(run, weights, launches)
-                if how.startswith("split"):
-                    # what the norm after it pays for reading the shares instead of one result (it runs one
-                    # workgroup a row; measured on MI355X at 64 rows of 4,096: 4 shares 3 µs, 8 shares 6.5 µs)
-                    times[how] += int(how[5:]) * rows * N * 4 / 1.5e12
         finally:
             self.product_plan = saved
         self._times[key] = dict(times)

@@ -338,7 +338,7 @@ def test_norm_finished_inside_the_products_around_it(ops, ref, M, H, K1, N2):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("R,H,S", [(5, 120, 2), (33, 1000, 4), (64, 4096, 8)])
+@pytest.mark.parametrize("R,H,S", [(5, 120, 2), (33, 1000, 4), (64, 4096, 8), (9, 5120, 4), (7, 8192, 8), (3, 8200, 2)])
 def test_add_rmsnorm_takes_a_product_in_shares(ops, ref, dtype, R, H, S):
     """The norm adds the shares of a product up in order, rounds the sum as the one product's result
     would have been rounded, and goes on as with that result; all rows, and a list of rows."""
@@ -360,7 +360,7 @@ def test_add_rmsnorm_takes_a_product_in_shares(ops, ref, dtype, R, H, S):
         torch.testing.assert_close(ha, hb, atol=1e-5, rtol=1e-5)
 
 
-@pytest.mark.parametrize("M", [8, 17, 64])
+@pytest.mark.parametrize("M", [8, 17, 64, 200, 600])
 def test_product_for_the_residual_stream_in_every_form(ops, monkeypatch, M):
     """linear_residual under every way the plan may name: bfloat16 rows or shares whose sum is the product."""
     from return_amd.parts.runtime import Slabs
@@ -373,7 +373,7 @@ def test_product_for_the_residual_stream_in_every_form(ops, monkeypatch, M):
     assert ("split4" in ways) == (M > 16) and "library" in ways
     for how in ways:
         plan.clear()
-        plan[(ops._rows_step(M), N, K, False, "residual")] = how
+        plan[(ops._rows_step(M, True), N, K, False, "residual")] = how
         y = ops.linear_residual(x, w)
         if how.startswith("split"):
             assert isinstance(y, Slabs) and tuple(y.tensor.shape) == (int(how[5:]), M, N) and y.tensor.dtype == torch.float32
@@ -459,6 +459,35 @@ def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
         assert plan.get(key) == choice and measured[key] == choice
     other = HipOps(DEV)
     assert other.product_plan == {} and other.route_linear(1, 768, 256, torch.bfloat16) == "skinny"
+
+
+def test_products_for_the_residual_stream_are_measured_at_some_hundred_rows_too(ops, monkeypatch):
+    """Beyond 64 rows only the products whose result goes into the residual stream are measured (the
+    library's one product against its batch over pieces of K, each with the norm that takes the result),
+    up to the rows a step can bring; other products of that many rows stay with the rule."""
+    plan, measured = {}, {}
+    monkeypatch.setattr(ops, "product_plan", plan)
+    monkeypatch.setattr(ops, "_measured", measured)
+    ws = [rnd(160, 2048, dtype=torch.bfloat16, seed=i, scale=0.1) for i in range(2)]
+    ops.tune_products([(w, False, "residual") for w in ws] + [(w, False, None) for w in ws], max_rows=2, max_rows_residual=200)
+    rows_res = {r for (r, N, K, gated, od) in measured if od == "residual"}
+    rows_plain = {r for (r, N, K, gated, od) in measured if od != "residual"}
+    assert rows_plain == {1, 2} and rows_res == {1, 2, 96, 128, 192, 256}
+    assert ops._rows_step(200, True) == 256 and ops._rows_step(200) == 0 and ops._rows_step(5000, True) == 0
+    for (rows, N, K, gated, od), how in plan.items():
+        assert how in ops._candidates(rows, N, K, gated, od)
+    # what the plan names at 256 rows is what 200 rows get, as shares or as rows; both give the product
+    x = rnd(200, 2048, dtype=torch.bfloat16, seed=5)
+    want = x.double() @ ws[0].double().t()
+    from return_amd.parts.runtime import Slabs
+    for how in ("library", "split2", "split8"):
+        plan[(256, 160, 2048, False, "residual")] = how
+        assert ops.route_linear(200, 160, 2048, "residual") == how
+        y = ops.linear_residual(x, ws[0])
+        got = y.tensor.double().sum(0) if isinstance(y, Slabs) else y.double()
+        assert isinstance(y, Slabs) == how.startswith("split")
+        torch.testing.assert_close(got, want, atol=0.3, rtol=2e-2)
+    assert ops.route_linear(200, 160, 2048, torch.bfloat16) == "library"
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
