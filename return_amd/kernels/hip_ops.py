@@ -364,7 +364,7 @@ class HipOps:
     # prompts beside decoded tokens) the library gives a product with few result columns and many of K too
     # few workgroups, and a batch over pieces of K is up to twice as fast (measured on MI355X, 512 rows:
     # 8B down 84 -> 55 µs, 32B down 272 -> 122 µs)
-    ROW_STEPS_RESIDUAL = (96, 128, 192, 256, 384, 512, 640, 768, 1024)
+    ROW_STEPS_RESIDUAL = (96, 128, 192, 256, 384, 512, 640, 768, 1024, 1536, 2048, 3072, 4096)
 
     def _rows_step(self, M, residual=False):
         for r in self.ROW_STEPS + (self.ROW_STEPS_RESIDUAL if residual else ()):
