@@ -675,7 +675,9 @@ class HipOps:
                     continue
                 key = (rows, N, K, gated, out_dtype)
                 if key not in self._measured:
-                    self._measured[key] = self._measure(key, uniq, launches, margin)
+                    # (products of many rows take long enough to be timed over a few launches)
+                    few = launches if rows <= self.ROW_STEPS[-1] else max(2, min(launches, 2048 // rows))
+                    self._measured[key] = self._measure(key, uniq, few, margin)
                 if self._measured[key] is not None:
                     self.product_plan[key] = self._measured[key]
 
