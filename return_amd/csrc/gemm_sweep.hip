@@ -218,7 +218,8 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_kernel(
 
 #define SW_SPAN (SW_WAVES * SW_KW)        // columns of K that the eight waves cover at once
 
-template <bool GATED, typename TO, bool RESID = false>
+// HELD: K is at most two spans, and the columns of x of both stay in registers for all tiles.
+template <bool GATED, typename TO, bool RESID = false, bool HELD = false>
 __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ W, TO* __restrict__ out, int M, int N, int K, SweepNorm nm) {
     static_assert(!RESID || !GATED, "the residual epilogue belongs to the plain product");
@@ -248,6 +249,16 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
     };
 #pragma unroll
     for (int i = 0; i < 16; ++i) fetch_row(0, 0, i);
+    [[maybe_unused]] bf16x8_t held[HELD ? 2 : 1][SW_STEPS];
+    if constexpr (HELD) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int j = 0; j < SW_STEPS; ++j) {
+                const int k = p * SW_SPAN + kb + 32 * j + 8 * g;
+                held[p][j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
+            }
+    }
     if (scaled) sweep_scales_make(nm, 16, share, rs);
     [[maybe_unused]] float sq = 0.f;
 
@@ -259,12 +270,17 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
             wn = nm.w_next[col];
         }
         float4_t c = {0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < spans; ++p) {
+#pragma unroll
+        for (int p = 0; p < (HELD ? 2 : spans); ++p) {
             bf16x8_t bx[SW_STEPS];                              // the span's columns of x as B operands
 #pragma unroll
             for (int j = 0; j < SW_STEPS; ++j) {
-                const int k = p * SW_SPAN + kb + 32 * j + 8 * g;
-                bx[j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
+                if constexpr (HELD) {
+                    bx[j] = held[p][j];
+                } else {
+                    const int k = p * SW_SPAN + kb + 32 * j + 8 * g;
+                    bx[j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
+                }
             }
             SW_WAVE_SYNC();
             const bool more = p + 1 < spans || t + 1 < n_tiles;
@@ -349,8 +365,12 @@ template <bool GATED, typename TO, bool RESID>
 static int launch_sweep(int grid, hipStream_t st, const bf16* x, const bf16* W, TO* out, int M, int N, int K,
                         const SweepNorm& nm) {
     if (K > SW_SPAN) {
+        if (K <= 2 * SW_SPAN) {
+            static bool allowed = false;
+            return launch_sweep_kernel(gemm_sweep_long_kernel<GATED, TO, RESID, true>, allowed, grid, st, x, W, out, M, N, K, nm);
+        }
         static bool allowed = false;
-        return launch_sweep_kernel(gemm_sweep_long_kernel<GATED, TO, RESID>, allowed, grid, st, x, W, out, M, N, K, nm);
+        return launch_sweep_kernel(gemm_sweep_long_kernel<GATED, TO, RESID, false>, allowed, grid, st, x, W, out, M, N, K, nm);
     }
     if constexpr (!RESID) {
         if (M > 16) {
