@@ -338,6 +338,131 @@ __global__ __launch_bounds__(SW_THREADS) void gemm_sweep_long_kernel(
     }
 }
 
+#define SW_FEW_TILES 4                    // tiles a workgroup has at most in gemm_sweep_spans_kernel
+
+// K beyond two spans and at most SW_FEW_TILES tiles a workgroup (few result columns, many of K: a down
+// projection): span by span, so that a span's columns of x are read once and serve every tile; the tiles'
+// sums stay in registers until the last span. (gemm_sweep_long_kernel reads x again for every tile, as many
+// bytes as the tile of W.)
+template <bool GATED, typename TO, bool RESID = false>
+__global__ __launch_bounds__(SW_THREADS) void gemm_sweep_spans_kernel(
+    const bf16* __restrict__ x, const bf16* __restrict__ W, TO* __restrict__ out, int M, int N, int K, SweepNorm nm) {
+    static_assert(!RESID || !GATED, "the residual epilogue belongs to the plain product");
+    constexpr int COLS = GATED ? 8 : 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    uint16_t* stage = reinterpret_cast<uint16_t*>(lds_raw) + (size_t)wave * 16 * SW_STRIDE;
+    float* red_both = reinterpret_cast<float*>(lds_raw + (size_t)SW_WAVES * 16 * SW_STRIDE * 2);
+    float* rs = red_both + 2 * SW_WAVES * 16 * 17;
+    const int G = gridDim.x, b = blockIdx.x;
+    const int my_cols = N > b ? (N - 1 - b) / G + 1 : 0;
+    const int n_tiles = (my_cols + COLS - 1) / COLS;          // (the launch keeps it within SW_FEW_TILES)
+    if (n_tiles == 0) return;
+    const int spans = (K + SW_SPAN - 1) / SW_SPAN;
+    const int kb = wave * SW_KW;
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    const bool scaled = nm.psq_in != nullptr;
+    float share[SW_SHARES];
+    if (scaled) sweep_scales_ask(nm, M, share);
+    bf16x8_t wreg[16];
+    auto fetch_row = [&](int t, int p, int i) {
+        const int k = p * SW_SPAN + kb + lane * 8;
+        const int col = b + G * (t * COLS + (GATED ? (i & 7) : i));
+        const size_t row = (GATED && i >= 8) ? (size_t)N + col : (size_t)col;
+        wreg[i] = (k < K && col < N) ? *reinterpret_cast<const bf16x8_t*>(W + row * K + k) : zero;
+    };
+#pragma unroll
+    for (int i = 0; i < 16; ++i) fetch_row(0, 0, i);
+    if (scaled) sweep_scales_make(nm, 16, share, rs);
+    float4_t c[SW_FEW_TILES];
+#pragma unroll
+    for (int t = 0; t < SW_FEW_TILES; ++t) c[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // RESID: the tiles' entries of h and of the next norm's weight are asked for at the start of the last
+    // span, before its rows of W (asked for in the epilogue they would be waited for; see the kernel above)
+    [[maybe_unused]] float h_old[SW_FEW_TILES], wn[SW_FEW_TILES];
+    for (int p = 0; p < spans; ++p) {
+        if constexpr (RESID) {
+            if (p == spans - 1) {
+#pragma unroll
+                for (int t = 0; t < SW_FEW_TILES; ++t) {
+                    const int mm = min(tid / COLS, M - 1), col = min(b + G * (min(t, n_tiles - 1) * COLS + tid % COLS), N - 1);
+                    h_old[t] = nm.h[(size_t)mm * N + col];
+                    wn[t] = nm.w_next[col];
+                }
+            }
+        }
+        bf16x8_t bx[SW_STEPS];                                  // the span's columns of x as B operands, for every tile
+#pragma unroll
+        for (int j = 0; j < SW_STEPS; ++j) {
+            const int k = p * SW_SPAN + kb + 32 * j + 8 * g;
+            bx[j] = (n < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(x + (size_t)n * K + k) : zero;
+        }
+#pragma unroll
+        for (int t = 0; t < SW_FEW_TILES; ++t) {
+            if (t >= n_tiles) break;
+            SW_WAVE_SYNC();
+            const bool more = t + 1 < n_tiles || p + 1 < spans;
+            const int t_next = t + 1 < n_tiles ? t + 1 : 0, p_next = t + 1 < n_tiles ? p : p + 1;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                *reinterpret_cast<bf16x8_t*>(&stage[i * SW_STRIDE + lane * 8]) = wreg[i];
+                if (more) fetch_row(t_next, p_next, i);
+            }
+            SW_WAVE_SYNC();
+#pragma unroll
+            for (int j = 0; j < SW_STEPS; ++j) {
+                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&stage[n * SW_STRIDE + 32 * j + 8 * g]);
+                c[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bx[j], c[t], 0, 0, 0);
+            }
+        }
+    }
+    MFMA_SETTLE();
+    [[maybe_unused]] float sq = 0.f;
+#pragma unroll
+    for (int t = 0; t < SW_FEW_TILES; ++t) {
+        if (t >= n_tiles) break;
+        float* red = red_both + (t & 1) * (SW_WAVES * 16 * 17);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[(wave * 16 + 4 * g + i) * 17 + n] = c[t][i];
+        __syncthreads();
+        if (tid < 16 * COLS) {
+            const int mm = tid / COLS, r = tid % COLS;
+            const int col = b + G * (t * COLS + r);
+            if (mm < M && col < N) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < SW_WAVES; ++w) s += red[(w * 16 + r) * 17 + mm];
+                const float scale = scaled ? rs[mm] : 1.0f;
+                s *= scale;
+                if constexpr (GATED) {
+                    float up = 0.f;
+#pragma unroll
+                    for (int w = 0; w < SW_WAVES; ++w) up += red[(w * 16 + 8 + r) * 17 + mm];
+                    s = s / (1.0f + expf(-s)) * (up * scale);
+                }
+                if constexpr (RESID) {
+                    const size_t at = (size_t)mm * N + col;
+                    const float hv = h_old[t] + round_to<bf16>(s);
+                    nm.h[at] = hv;
+                    out[at] = from_f<TO>(hv * wn[t]);
+                    sq += hv * hv;
+                } else {
+                    out[(size_t)mm * N + col] = from_f<TO>(s);
+                }
+            }
+        }
+    }
+    if constexpr (RESID) {
+        if (tid < 16 * COLS) {
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 16);
+            if ((tid & 15) == 0 && (tid >> 4) < M) nm.psq_out[(size_t)(tid >> 4) * G + b] = sq;
+        }
+    }
+}
+
 // the waves' W tiles, and their result tiles: two sets of 17 columns or one of 33
 static size_t sweep_lds() { return (size_t)SW_WAVES * 16 * SW_STRIDE * 2 + (size_t)2 * SW_WAVES * 16 * 17 * 4 + 32 * 4; }
 
@@ -368,6 +493,12 @@ static int launch_sweep(int grid, hipStream_t st, const bf16* x, const bf16* W, 
         if (K <= 2 * SW_SPAN) {
             static bool allowed = false;
             return launch_sweep_kernel(gemm_sweep_long_kernel<GATED, TO, RESID, true>, allowed, grid, st, x, W, out, M, N, K, nm);
+        }
+        const int cols = GATED ? 8 : 16, workgroups = grid < N ? grid : N;
+        const int most_tiles = ((N + workgroups - 1) / workgroups + cols - 1) / cols;
+        if (most_tiles >= 2 && most_tiles <= SW_FEW_TILES) {    // (with one tile the two orders are the same, and this one a little slower)
+            static bool allowed = false;
+            return launch_sweep_kernel(gemm_sweep_spans_kernel<GATED, TO, RESID>, allowed, grid, st, x, W, out, M, N, K, nm);
         }
         static bool allowed = false;
         return launch_sweep_kernel(gemm_sweep_long_kernel<GATED, TO, RESID, false>, allowed, grid, st, x, W, out, M, N, K, nm);
