@@ -556,35 +556,48 @@ extern "C" int ra_dec_part_1(DEC_PART_ARGS);
 extern "C" int ra_dec_part_2(DEC_PART_ARGS);
 extern "C" int ra_dec_part_3(DEC_PART_ARGS);
 
-// Merge of the splits, in split order: out = sum_s acc_s * w_s / sum_s l_s * w_s, w_s = exp(m_s - m).
+// Merge of the splits: out = sum_s acc_s * w_s / sum_s l_s * w_s, w_s = exp(m_s - m).
 // The kernel is a chain of loads that wait for each other (the request's tables, then the splits'
 // maxima, then their sums), and each link costs about a microsecond after a kernel that wrote them.
-// So the first COMBINE_AHEAD splits' maxima and sums are asked for at once with the tables, before it
+// So a thread's COMBINE_AHEAD splits' maxima and sums are asked for at once with the tables, before it
 // is known how many splits hold keys: what a split beyond them left in memory is read and not used.
-// Every thread forms the weights itself (the same numbers in the same order), so that no thread waits
-// for another.
+// A request of more than COMBINE_AHEAD splits has GROUPS groups of 128 threads, each for a run of
+// at most COMBINE_AHEAD consecutive splits (or more, by a loop, beyond 8 groups' worth), so that all
+// loads of a long request are on their way together; the groups' sums are merged through LDS in group
+// order. Every thread forms the weights itself (the same numbers in the same order), so that within a
+// group no thread waits for another.
 #define COMBINE_AHEAD 16
-__global__ __launch_bounds__(128) void attn_decode_combine_kernel(
+#define COMBINE_MAX_GROUPS 8
+template <int GROUPS>
+__global__ __launch_bounds__(128 * GROUPS) void attn_decode_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
     const int* __restrict__ kv_start, const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ seg_ids, int Hq, int D, int window, int split_tokens, int max_splits) {
-    const int di = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
-    const float* pm = part_ml + ((size_t)di * Hq + head) * max_splits * 2;
-    const float* pa = part_acc + ((size_t)di * Hq + head) * max_splits * D;
+    const int di = blockIdx.x, head = blockIdx.y, tid = threadIdx.x & 127, grp = threadIdx.x >> 7;
+    // this group's run of splits: [first, first + per)
+    const int per = GROUPS == 1 ? max_splits : (max_splits + GROUPS - 1) / GROUPS;
+    const int first = grp * per;
+    const float* pm = part_ml + (((size_t)di * Hq + head) * max_splits + first) * 2;
+    const float* pa = part_acc + (((size_t)di * Hq + head) * max_splits + first) * D;
     const int d0 = min(tid, D - 1), d1 = min(tid + 128, D - 1);       // this thread's columns (D <= 256), clamped for the loads
     float2_t ml[COMBINE_AHEAD];
     float a0[COMBINE_AHEAD], a1[COMBINE_AHEAD];
+    const int last_valid = max(max_splits - 1 - first, 0);           // (a group beyond the splits reads the last one and uses nothing)
+    const bool any = first < max_splits;
 #pragma unroll
     for (int s = 0; s < COMBINE_AHEAD; ++s) {
-        const int sc = min(s, max_splits - 1);
-        ml[s] = *reinterpret_cast<const float2_t*>(pm + 2 * sc);
-        a0[s] = pa[(size_t)sc * D + d0];
-        a1[s] = pa[(size_t)sc * D + d1];
+        const int sc = any ? min(s, last_valid) : 0;
+        const float* pms = any ? pm : part_ml + ((size_t)di * Hq + head) * max_splits * 2;
+        const float* pas = any ? pa : part_acc + ((size_t)di * Hq + head) * max_splits * D;
+        ml[s] = *reinterpret_cast<const float2_t*>(pms + 2 * sc);
+        a0[s] = pas[(size_t)sc * D + d0];
+        a1[s] = pas[(size_t)sc * D + d1];
     }
     const int seg = seg_ids ? seg_ids[di] : di;
     const int t = cu_q ? cu_q[seg] : seg;
     const DecodeRange rg = decode_range(q_start[seg], kv_start[seg], window, split_tokens, 0);
-    const int ns = min(rg.n_splits, max_splits);
+    const int ns_all = min(rg.n_splits, max_splits);
+    const int ns = max(0, min(ns_all - first, per));        // splits of this group that hold keys
     float m = -INFINITY;                                   // (the maxima are base-2 exponents)
 #pragma unroll
     for (int s = 0; s < COMBINE_AHEAD; ++s) m = s < ns ? fmaxf(m, ml[s][0]) : m;
@@ -606,6 +619,25 @@ __global__ __launch_bounds__(128) void attn_decode_combine_kernel(
         l += pm[2 * s + 1] * w;
         o0 = fmaf(pa[(size_t)s * D + d0], w, o0);
         o1 = fmaf(pa[(size_t)s * D + d1], w, o1);
+    }
+    if constexpr (GROUPS > 1) {
+        // the groups' (m, l, o0, o1) per thread, merged by group 0 in group order
+        __shared__ float4_t sums[GROUPS][128];
+        sums[grp][tid] = float4_t{m, l, o0, o1};
+        __syncthreads();
+        if (grp != 0) return;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int g2 = 0; g2 < GROUPS; ++g2) mx = fmaxf(mx, sums[g2][tid][0]);
+        l = 0.f; o0 = 0.f; o1 = 0.f;
+#pragma unroll
+        for (int g2 = 0; g2 < GROUPS; ++g2) {
+            const float4_t v = sums[g2][tid];
+            const float w = (v[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(v[0] - mx);
+            l = fmaf(v[1], w, l);
+            o0 = fmaf(v[2], w, o0);
+            o1 = fmaf(v[3], w, o1);
+        }
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     bf16* o = out + ((size_t)t * Hq + head) * D;
@@ -658,8 +690,14 @@ static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const 
     if (rc != RA_OK) return rc;
     if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
     if (merge) return RA_OK;
-    hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_dec, Hq), dim3(128), 0, st, pa, pm, (bf16*)out, kv_start, cu_q,
-                       q_start, seg_ids, Hq, D, window, split_tokens, max_splits);
+#define DEC_COMBINE(G) hipLaunchKernelGGL(attn_decode_combine_kernel<G>, dim3(n_dec, Hq), dim3(128 * G), 0, st, pa, pm, \
+                                          (bf16*)out, kv_start, cu_q, q_start, seg_ids, Hq, D, window, split_tokens, max_splits)
+    const int groups = (max_splits + COMBINE_AHEAD - 1) / COMBINE_AHEAD;
+    if (groups <= 1) DEC_COMBINE(1);
+    else if (groups <= 2) DEC_COMBINE(2);
+    else if (groups <= 4) DEC_COMBINE(4);
+    else DEC_COMBINE(COMBINE_MAX_GROUPS);
+#undef DEC_COMBINE
     return ra_launch_status();
 }
 
