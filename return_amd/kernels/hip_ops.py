@@ -676,7 +676,7 @@ class HipOps:
                 key = (rows, N, K, gated, out_dtype)
                 if key not in self._measured:
                     # (products of many rows take long enough to be timed over a few launches)
-                    few = launches if rows <= self.ROW_STEPS[-1] else max(2, min(launches, 2048 // rows))
+                    few = launches if rows <= self.ROW_STEPS[-1] else max(4, min(launches, 4096 // rows))
                     self._measured[key] = self._measure(key, uniq, few, margin)
                 if self._measured[key] is not None:
                     self.product_plan[key] = self._measured[key]
