@@ -348,19 +348,29 @@ def contexts_8b(args):
             got = step_bytes / (ms * 1e-3) / 1e9
             points[f"decode_b{b}_ctx{ctx}"] = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4),
                                               "GBs": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4)}
-    # ---- sampling at 64 rows of the full vocabulary: greedy against temperature 1 with top_p 0.9
-    logits = torch.randn(64, cfg.vocab_size, device="cuda:0") * 3.0
+    # ---- sampling at 64 rows of the full vocabulary: greedy, temperature 1 alone, with top_p 0.9, with top_k 50;
+    # on flat rows (N(0, 3): thresholds are searched over the whole row) and on rows shaped like a language
+    # model's (a bulk of N(0, 1.5), 500 tokens at 10 to 20 and one at 24: thresholds from the list of the largest)
+    gen = torch.Generator(device="cuda:0").manual_seed(5)
+    flat = torch.randn(64, cfg.vocab_size, device="cuda:0", generator=gen) * 3.0
+    peaked = torch.randn(64, cfg.vocab_size, device="cuda:0", generator=gen) * 1.5
+    for r in range(64):
+        idx = torch.randperm(cfg.vocab_size, device="cuda:0", generator=gen)[:500]
+        peaked[r, idx] = 10.0 + 10.0 * torch.rand(500, device="cuda:0", generator=gen)
+        peaked[r, idx[0]] = 24.0
     sampling = {}
-    for name, temp, top_p in (("greedy", 0.0, 1.0), ("top_p_0.9", 1.0, 0.9), ("top_k_50", 1.0, 1.0)):
-        best = None
-        for _ in range(5):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            runner.sample(logits, [temp] * 64, [50 if name == "top_k_50" else 0] * 64, [top_p] * 64, [0.37] * 64)
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-        sampling[name + "_us"] = round(best * 1e6, 1)
-    del logits
+    for prefix, logits in (("", flat), ("peaked_", peaked)):
+        for name, temp, top_p in (("greedy", 0.0, 1.0), ("temperature_1", 1.0, 1.0), ("top_p_0.9", 1.0, 0.9),
+                                  ("top_k_50", 1.0, 1.0)):
+            best = None
+            for _ in range(5):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                runner.sample(logits, [temp] * 64, [50 if name == "top_k_50" else 0] * 64, [top_p] * 64, [0.37] * 64)
+                dt = time.perf_counter() - t0
+                best = dt if best is None else min(best, dt)
+            sampling[prefix + name + "_us"] = round(best * 1e6, 1)
+    del flat, peaked
     # ---- one prompt of 16,384 tokens in one portion
     n = 16384
     del runner

@@ -10,10 +10,23 @@
 // The draw uses a uniform number u in [0,1) that the host supplies per row: the token is the
 // first, in vocabulary order, at which the running sum of kept probabilities exceeds u.
 // Tokens that tie with the k-th value, or with the top-p boundary value, are all kept.
+//
+// top-k and top-p need a threshold among the largest logits. The row's tokens within CAND_SPAN of
+// the largest logit (in units of the temperature: every other token weighs less than e^-16 of the
+// largest) are first collected into a list in LDS, in vocabulary order; if they fit, and if the
+// thresholds lie among them (k is at most their number; their mass is more than top_p of the whole),
+// the thresholds are searched and the token is drawn from the list alone, which takes microseconds.
+// Otherwise (a flat row, a large k, top_p near 1) the searches go over the whole row, pass by pass.
+// Which way a row goes depends on that row alone.
 #include "common.h"
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_BUCKETS 32
+#define CAND_WAVES (SAMPLE_THREADS / 64)
+#define CAND_PER_WAVE 512                                        // list entries of one wave's run of the row
+#define CAND_OWN (CAND_WAVES * CAND_PER_WAVE / SAMPLE_THREADS)   // entries a thread looks after in a search: 8
+#define CAND_SPAN 16.0f
+#define SAMPLE_BLOCKS 64                                         // blocks of 256 tokens in a wave's run whose masses are kept
 
 __device__ __forceinline__ uint32_t order_key(float f) {
     const uint32_t b = __float_as_uint(f);
@@ -46,6 +59,23 @@ __device__ __forceinline__ void for_each_logit(const float* __restrict__ x, int 
     }
 }
 
+// One thread's end of a pass of the threshold search: tot[b] is the measure of run b of (lo, hi], cut into
+// nb runs of 2^sh keys. Run b ends at key T_b = lo + ((b + 1) << sh) - 1; the measure above T_b is above_hi
+// plus the runs above b. The threshold lies in the lowest run whose end has at most `limit` above it.
+__device__ __forceinline__ void narrow_range(uint32_t lo, uint32_t hi, int sh, int nb, float above_hi, float limit,
+                                             const float* tot, uint32_t* sh_range, float* sh_above) {
+    float above = above_hi;
+    int b = nb - 1;
+    while (b > 0 && above + tot[b] <= limit) {
+        above += tot[b];
+        --b;
+    }
+    const unsigned long long end = (unsigned long long)lo + (((unsigned long long)b + 1ull) << sh) - 1ull;
+    sh_range[1] = end < (unsigned long long)hi ? (uint32_t)end : hi;
+    sh_range[0] = b == 0 ? lo : lo + ((uint32_t)b << sh);   // the run below ends with more than `limit` above it
+    sh_above[0] = above;
+}
+
 // The smallest key t in [lo, hi] with measure{key > t} <= limit, where the measure of a token is 1
 // (MASS false: counts, exact in 32-bit floats below 2^24) or exp((x - gmax) * inv_t) (MASS true), and
 // measure{key > hi} = above_hi <= limit. Every pass over the row cuts [lo, hi] into up to 32 runs of
@@ -66,7 +96,7 @@ __device__ uint32_t find_threshold(const float* __restrict__ x, int V, int tid, 
         for_each_logit(x, V, tid, [&](int, float v) {
             const uint32_t key = order_key(v);
             if (key > lo && key <= hi) {
-                const float w = MASS ? expf((v - gmax) * inv_t) : 1.0f;
+                const float w = MASS ? __expf((v - gmax) * inv_t) : 1.0f;
                 bins[((key - lo) >> sh) * SAMPLE_THREADS + tid] += w;
             }
         });
@@ -86,20 +116,73 @@ __device__ uint32_t find_threshold(const float* __restrict__ x, int V, int tid, 
             tot[tid] = t;
         }
         __syncthreads();
-        if (tid == 0) {
-            // run b ends at key T_b = lo + ((b + 1) << sh) - 1; the measure above T_b is above_hi plus the
-            // runs above b. t lies in the lowest run whose end has at most `limit` above it.
-            float above = above_hi;
-            int b = nb - 1;
-            while (b > 0 && above + tot[b] <= limit) {
-                above += tot[b];
-                --b;
-            }
-            const unsigned long long end = (unsigned long long)lo + (((unsigned long long)b + 1ull) << sh) - 1ull;
-            sh_range[1] = end < (unsigned long long)hi ? (uint32_t)end : hi;
-            sh_range[0] = b == 0 ? lo : lo + ((uint32_t)b << sh);   // the run below ends with more than `limit` above it
-            sh_above[0] = above;
+        if (tid == 0) narrow_range(lo, hi, sh, nb, above_hi, limit, tot, sh_range, sh_above);
+        __syncthreads();
+        lo = sh_range[0];
+        hi = sh_range[1];
+        above_hi = sh_above[0];
+        __syncthreads();
+    }
+    return lo;
+}
+
+// The draw's first step: wmass[w] is the kept mass of wave w's run of tokens (runs in vocabulary order).
+// Gives the wave in whose run the running sum passes u times the total (the last run with kept mass if it
+// never does), the sum before that run and the target. Every thread computes the same.
+__device__ __forceinline__ void pick_wave(const float* wmass, float u, int& owner, float& before, float& target) {
+    float total = 0.f;
+    for (int w = 0; w < CAND_WAVES; ++w) total += wmass[w];
+    target = u * total;
+    float run = 0.f;
+    owner = -1;
+    before = 0.f;
+    for (int w = 0; w < CAND_WAVES; ++w) {
+        if (wmass[w] > 0.f) {
+            owner = w;
+            before = run;
+            if (run + wmass[w] > target) break;
+            run += wmass[w];
         }
+    }
+}
+
+// Running sums over the lanes of a wave, lane by lane in lane order (inclusive).
+__device__ __forceinline__ float wave_running_sum(float v, int lane) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float t = __shfl_up(v, o, 64);
+        if (lane >= o) v += t;
+    }
+    return v;
+}
+
+// find_threshold over the list instead of the row: a thread holds CAND_OWN entries (key 0 where the list
+// has none). The measure of a run is added up in whole numbers, a token's weight as a multiple of 2^-40
+// (1 for counts), by LDS atomics: such sums do not depend on the order in which they are formed, so the
+// result is the same in every run of the program. fx: [SAMPLE_BUCKETS] 64-bit words of LDS.
+#define LIST_ONE 1099511627776.0f                  // 2^40
+template <bool MASS>
+__device__ uint32_t list_threshold(const uint32_t (&key)[CAND_OWN], const float (&weight)[CAND_OWN], int tid,
+                                   uint32_t lo, uint32_t hi, float limit, unsigned long long* fx, float* tot,
+                                   uint32_t* sh_range, float* sh_above) {
+    unsigned long long wfx[CAND_OWN];
+#pragma unroll
+    for (int e = 0; e < CAND_OWN; ++e) wfx[e] = MASS ? (unsigned long long)(weight[e] * LIST_ONE + 0.5f) : (1ull << 40);
+    float above_hi = 0.f;
+    while (lo < hi) {
+        const uint32_t width = hi - lo;
+        const int bits = 32 - __builtin_clz(width);
+        const int sh = bits > 5 ? bits - 5 : 0;
+        const int nb = (int)(width >> sh) + 1;
+        if (tid < SAMPLE_BUCKETS) fx[tid] = 0ull;
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < CAND_OWN; ++e)
+            if (key[e] > lo && key[e] <= hi) atomicAdd(&fx[(key[e] - lo) >> sh], wfx[e]);
+        __syncthreads();
+        if (tid < SAMPLE_BUCKETS) tot[tid] = (float)fx[tid] * (1.0f / LIST_ONE);
+        __syncthreads();
+        if (tid == 0) narrow_range(lo, hi, sh, nb, above_hi, limit, tot, sh_range, sh_above);
         __syncthreads();
         lo = sh_range[0];
         hi = sh_range[1];
@@ -112,13 +195,14 @@ __device__ uint32_t find_threshold(const float* __restrict__ x, int V, int tid, 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ u,
-    int* __restrict__ out) {
+    int* __restrict__ out, int* __restrict__ path) {
     extern __shared__ __attribute__((aligned(16))) float bins[];          // [SAMPLE_BUCKETS][SAMPLE_THREADS]
     __shared__ float scratch[16];
     __shared__ float part[SAMPLE_THREADS];
     __shared__ float tot[SAMPLE_BUCKETS];
     __shared__ uint32_t sh_range[2];
-    __shared__ int sh_int[4];
+    __shared__ float wmass[CAND_WAVES];
+    __shared__ unsigned long long fx[SAMPLE_BUCKETS];
     __shared__ float sh_f[2];
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* x = logits + (size_t)row * V;
@@ -167,79 +251,300 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         if (tid == 0) {
             out[2 * row] = argmax;
             out[2 * row + 1] = __float_as_int(x[argmax] - lse);
+            if (path) path[row] = 0;
         }
         return;
     }
     const float inv_t = 1.0f / temp;
     const uint32_t top_key = order_key(gmax);
 
-    // ---- top-k: the key of the k-th largest value is the smallest key with at most k - 1 tokens above it
-    uint32_t keep_key = 0u;                   // keep tokens whose key >= keep_key
+    // Wave w's run of the row (a multiple of 256 tokens): a lane reads four consecutive tokens of every 256,
+    // so that what a wave meets, load by load, lane by lane, is in vocabulary order.
+    const int wave = tid >> 6, lane = tid & 63;
+    const int seg = ((V + CAND_WAVES - 1) / CAND_WAVES + 255) / 256 * 256;
+    const int beg = min(V, wave * seg), end = min(V, beg + seg);
+    const bool vec = (V & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    auto load4 = [&](int i, float (&a)[4]) {           // tokens i .. i+3 of the run, -inf beyond its end
+        if (vec) {
+            if (i < end) {
+                const float4 t = *reinterpret_cast<const float4*>(x + i);
+                a[0] = t.x; a[1] = t.y; a[2] = t.z; a[3] = t.w;
+            } else {
+                a[0] = a[1] = a[2] = a[3] = -INFINITY;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) a[c] = i + c < end ? x[i + c] : -INFINITY;
+        }
+    };
+
     const int k = top_k[row];
-    if (k > 0 && k < V)
-        keep_key = find_threshold<false>(x, V, tid, 0u, top_key, 0.f, (float)(k - 1), gmax, inv_t, bins, part, tot,
-                                         sh_range, sh_f);
-
-    // ---- top-p: the smallest key with at most p of the kept mass above it
     const float p = top_p[row];
-    if (p < 1.0f) {
-        float z = 0.f;
-        for_each_logit(x, V, tid, [&](int, float v) {
-            if (order_key(v) >= keep_key) z += expf((v - gmax) * inv_t);
-        });
-        z = block_sum(z, scratch);
-        keep_key = find_threshold<true>(x, V, tid, keep_key, top_key, 0.f, p * z, gmax, inv_t, bins, part, tot,
-                                        sh_range, sh_f);
+    const bool want_k = k > 0 && k < V, want_p = p < 1.0f;
+    uint32_t keep_key = 0u;                   // keep tokens whose key >= keep_key
+
+    if (want_k || want_p) {
+        // ---- the list: wave w goes through its run of the row, 64 tokens a load, and appends the tokens
+        // within CAND_SPAN of the largest to its part of the list, in their order
+        float* cv = bins;                                                  // [CAND_WAVES][CAND_PER_WAVE] logits
+        int* ci = reinterpret_cast<int*>(bins + CAND_WAVES * CAND_PER_WAVE);   // and their token numbers
+        __shared__ int cnt[CAND_WAVES];
+        __shared__ int sh_over;
+        const float cut = gmax - CAND_SPAN * temp;
+        const uint32_t cut_key = order_key(cut);
+        const bool sum_rest = want_p && !want_k;       // top-p alone is over the mass of the whole row
+        if (tid == 0) sh_over = 0;
+        __syncthreads();
+        {
+            int have = 0;
+            float rest = 0.f;
+            const unsigned long long below = (1ull << lane) - 1ull;        // the lanes before this one
+            for (int i0 = beg + 4 * lane; i0 - 4 * lane < end; i0 += 4 * 256) {      // four loads on their way
+                float v[4][4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) load4(i0 + 256 * j, v[j]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    int before = 0, all = 0;
+                    bool in[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        in[c] = v[j][c] >= cut;
+                        const unsigned long long m = __ballot(in[c]);
+                        before += __popcll(m & below);
+                        all += __popcll(m);
+                    }
+                    if (all != 0) {
+                        int at = have + before;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            if (in[c]) {
+                                if (at < CAND_PER_WAVE) {
+                                    cv[wave * CAND_PER_WAVE + at] = v[j][c];
+                                    ci[wave * CAND_PER_WAVE + at] = i0 + 256 * j + c;
+                                }
+                                ++at;
+                            }
+                        }
+                        have += all;
+                    }
+                    if (sum_rest) {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) rest += in[c] ? 0.f : __expf((v[j][c] - gmax) * inv_t);
+                    }
+                }
+            }
+            if (lane == 0) {
+                cnt[wave] = min(have, CAND_PER_WAVE);
+                if (have > CAND_PER_WAVE) sh_over = 1;
+            }
+            const float z_rest = sum_rest ? block_sum(rest, scratch) : 0.f;     // (with barriers of its own, or:)
+            __syncthreads();
+            int total = 0;
+            for (int w = 0; w < CAND_WAVES; ++w) total += cnt[w];
+            bool listed = sh_over == 0 && cut_key > 0u && (!want_k || k <= total);
+
+            // a thread's entries for the searches: place (tid % CAND_PER_WAVE) of every other wave's part
+            uint32_t key[CAND_OWN];
+            float weight[CAND_OWN];
+            if (listed) {
+                const int half = tid / CAND_PER_WAVE, off = tid - half * CAND_PER_WAVE;
+#pragma unroll
+                for (int e = 0; e < CAND_OWN; ++e) {
+                    const int w = half + (SAMPLE_THREADS / CAND_PER_WAVE) * e;
+                    const bool there = off < cnt[w];
+                    const float v = there ? cv[w * CAND_PER_WAVE + off] : 0.f;
+                    key[e] = there ? order_key(v) : 0u;
+                    weight[e] = there ? __expf((v - gmax) * inv_t) : 0.f;
+                }
+                // top-k: the k-th largest is on the list; below cut_key - 1 nothing of it lies
+                if (want_k)
+                    keep_key = list_threshold<false>(key, weight, tid, cut_key - 1u, top_key, (float)(k - 1), fx, tot,
+                                                     sh_range, sh_f);
+                if (want_p) {
+                    float zc = 0.f;
+#pragma unroll
+                    for (int e = 0; e < CAND_OWN; ++e) zc += key[e] >= keep_key && key[e] != 0u ? weight[e] : 0.f;
+                    zc = block_sum(zc, scratch);
+                    const float z = zc + z_rest;
+                    // the boundary is on the list if the list's mass is more than p of the whole (always, after top-k)
+                    if (want_k || zc > p * z) {
+                        const uint32_t lo = want_k ? keep_key : cut_key - 1u;
+                        keep_key = list_threshold<true>(key, weight, tid, lo, top_key, p * z, fx, tot, sh_range, sh_f);
+                    } else {
+                        listed = false;
+                    }
+                }
+            }
+            if (listed) {
+                // ---- the draw over the list, which is in vocabulary order: wave w has its own part,
+                // a lane CAND_PER_WAVE / 64 consecutive entries of it
+                constexpr int RUN = CAND_PER_WAVE / 64;
+                const int o0 = min(cnt[wave], RUN * lane), o1 = min(cnt[wave], o0 + RUN);
+                float mine = 0.f;
+                for (int o = o0; o < o1; ++o) {
+                    const float v = cv[wave * CAND_PER_WAVE + o];
+                    if (order_key(v) >= keep_key) mine += __expf((v - gmax) * inv_t);
+                }
+                const float upto = wave_running_sum(mine, lane);
+                __syncthreads();
+                if (lane == 63) wmass[wave] = upto;
+                __syncthreads();
+                int owner;
+                float before, target;
+                pick_wave(wmass, u[row], owner, before, target);
+                if (owner < 0) {                       // (nothing is kept: cannot be, the largest always is)
+                    if (tid == 0) {
+                        out[2 * row] = argmax;
+                        out[2 * row + 1] = __float_as_int(x[argmax] - lse);
+                        if (path) path[row] = 1;
+                    }
+                    return;
+                }
+                if (wave != owner) return;
+                // the lane in whose entries the running sum passes the target, else the last one with kept mass
+                const unsigned long long passed = __ballot(mine > 0.f && before + upto > target);
+                const unsigned long long any = __ballot(mine > 0.f);
+                const int who = passed ? __ffsll((long long)passed) - 1 : 63 - __builtin_clzll(any);
+                if (lane == who) {
+                    float run = before + (upto - mine);
+                    int tok = argmax;
+                    for (int o = o0; o < o1; ++o) {
+                        const float v = cv[wave * CAND_PER_WAVE + o];
+                        if (order_key(v) >= keep_key) {
+                            tok = ci[wave * CAND_PER_WAVE + o];      // the last kept entry if the target is never passed
+                            run += __expf((v - gmax) * inv_t);
+                            if (run > target) break;
+                        }
+                    }
+                    out[2 * row] = tok;
+                    out[2 * row + 1] = __float_as_int(x[tok] - lse);
+                    if (path) path[row] = 1;
+                }
+                return;
+            }
+        }
+        __syncthreads();
+        keep_key = 0u;
+
+        // ---- over the whole row. top-k: the key of the k-th largest value is the smallest key with at most
+        // k - 1 tokens above it
+        if (want_k)
+            keep_key = find_threshold<false>(x, V, tid, 0u, top_key, 0.f, (float)(k - 1), gmax, inv_t, bins, part, tot,
+                                             sh_range, sh_f);
+        // top-p: the smallest key with at most p of the kept mass above it
+        if (want_p) {
+            float z = 0.f;
+            for_each_logit(x, V, tid, [&](int, float v) {
+                if (order_key(v) >= keep_key) z += __expf((v - gmax) * inv_t);
+            });
+            z = block_sum(z, scratch);
+            keep_key = find_threshold<true>(x, V, tid, keep_key, top_key, 0.f, p * z, gmax, inv_t, bins, part, tot,
+                                            sh_range, sh_f);
+        }
     }
 
-    // ---- inverse CDF in vocabulary order: contiguous chunk per thread
-    const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-    const int i0 = min(V, tid * chunk), i1 = min(V, i0 + chunk);
-    float mine = 0.f;
-    for (int i = i0; i < i1; ++i)
-        if (order_key(x[i]) >= keep_key) mine += expf((x[i] - gmax) * inv_t);
-    __syncthreads();
-    part[tid] = mine;
-    __syncthreads();
-    if (tid == 0) {
-        float total = 0.f;
-        for (int i = 0; i < SAMPLE_THREADS; ++i) total += part[i];
-        const float target = u[row] * total;
-        float run = 0.f, before = 0.f;
-        int owner = -1;
-        for (int i = 0; i < SAMPLE_THREADS; ++i) {
-            if (part[i] > 0.f) {
-                owner = i;                           // the last chunk with kept mass if the target is never passed
-                before = run;
-                if (run + part[i] > target) break;
-                run += part[i];
+    // ---- the draw over the whole row, in vocabulary order. Wave w has a run of the row (a multiple of 256
+    // tokens); a lane reads four consecutive tokens of every 256. First the kept mass of every block of 256
+    // tokens, and with them every wave's; then the wave in whose run the running sum passes the target finds
+    // the block in which it does, and goes through that block again, token by token.
+    {
+        auto kept_mass = [&](int i, float v) {             // (a token beyond the run's end has none: exp(-inf))
+            return (i < end && order_key(v) >= keep_key) ? __expf((v - gmax) * inv_t) : 0.f;
+        };
+        __shared__ float bmass[CAND_WAVES][SAMPLE_BLOCKS];
+        const int n_it = (end - beg + 255) / 256;            // this wave's blocks
+        const bool by_block = seg / 256 <= SAMPLE_BLOCKS;    // (a vocabulary beyond 262,144: the whole run is gone through again)
+        float mine = 0.f;
+        for (int it0 = 0; it0 < n_it; it0 += 4) {            // four loads on their way
+            float a[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load4(beg + 256 * (it0 + j) + 4 * lane, a[j]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = beg + 256 * (it0 + j) + 4 * lane;
+                float m = 0.f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) m += kept_mass(i + c, a[j][c]);
+                m = wave_sum(m);
+                if (by_block && lane == 0 && it0 + j < n_it) bmass[wave][it0 + j] = m;
+                mine += m;
             }
         }
-        sh_int[3] = owner < 0 ? 0 : owner;
-        sh_f[0] = before;
-        sh_f[1] = target;
-    }
-    __syncthreads();
-    if (tid == sh_int[3]) {
-        float run = sh_f[0];
-        const float target = sh_f[1];
-        int tok = -1;
-        for (int i = i0; i < i1; ++i) {
-            if (order_key(x[i]) >= keep_key) {
-                tok = i;                             // last kept token of the chunk if never passed
-                run += expf((x[i] - gmax) * inv_t);
-                if (run > target) break;
+        __syncthreads();
+        if (lane == 0) wmass[wave] = mine;
+        __syncthreads();
+        int owner;
+        float before, target;
+        pick_wave(wmass, u[row], owner, before, target);
+        if (owner < 0) owner = 0;
+        if (wave != owner) return;
+        float run = before;
+        int it_lo = 0, it_hi = n_it;
+        if (by_block) {                                      // the block, as pick_wave finds the wave
+            int ob = -1;
+            float r2 = before;
+            for (int it = 0; it < n_it; ++it) {
+                const float bm = bmass[wave][it];
+                if (bm > 0.f) {
+                    ob = it;
+                    run = r2;
+                    if (r2 + bm > target) break;
+                    r2 += bm;
+                }
+            }
+            it_lo = max(ob, 0);
+            it_hi = ob < 0 ? 0 : ob + 1;
+        }
+        int last_kept = -1, tok = -1;
+        constexpr int AHEAD = 4;                             // loads on their way
+        float a[AHEAD][4];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) load4(beg + 256 * (it_lo + j) + 4 * lane, a[j]);
+        for (int it0 = it_lo; it0 < it_hi && tok < 0; it0 += AHEAD) {
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) {
+                const int i = it0 + j < it_hi ? beg + 256 * (it0 + j) + 4 * lane : end;      // (beyond the blocks asked for: nothing)
+                float m[4], s[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) m[c] = kept_mass(i + c, a[j][c]);
+                s[0] = m[0]; s[1] = s[0] + m[1]; s[2] = s[1] + m[2]; s[3] = s[2] + m[3];
+                const float upto = wave_running_sum(s[3], lane);
+                const float base = run + (upto - s[3]);
+                int first = -1;
+#pragma unroll
+                for (int c = 3; c >= 0; --c) {
+                    const bool is_kept = i + c < end && order_key(a[j][c]) >= keep_key;
+                    if (is_kept && base + s[c] > target) first = c;
+                    if (is_kept) last_kept = max(last_kept, i + c);
+                }
+                const unsigned long long passed = __ballot(first >= 0);
+                if (passed && tok < 0) {
+                    const int who = __ffsll((long long)passed) - 1;
+                    tok = __shfl(i + max(first, 0), who, 64);
+                }
+                run += __shfl(upto, 63, 64);
+                load4(beg + 256 * (it0 + j + AHEAD) + 4 * lane, a[j]);                 // (beyond the run's end: -inf)
             }
         }
-        if (tok < 0) tok = argmax;
-        out[2 * row] = tok;
-        out[2 * row + 1] = __float_as_int(x[tok] - lse);
+        if (tok < 0) {                                       // never passed: the last kept token of the run
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) last_kept = max(last_kept, __shfl_xor(last_kept, o, 64));
+            tok = last_kept < 0 ? argmax : last_kept;
+        }
+        if (lane == 0) {
+            out[2 * row] = tok;
+            out[2 * row + 1] = __float_as_int(x[tok] - lse);
+            if (path) path[row] = (want_k || want_p) ? 2 : 0;
+        }
     }
 }
 
-extern "C" int ra_sample(const float* logits, int M, int V, const float* temperature,
-                         const int* top_k, const float* top_p, const float* u, int* out,
-                         void* stream) {
+// path (may be nullptr): per row 0 = no threshold was needed, 1 = thresholds and draw from the list of the
+// largest logits, 2 = by passes over the whole row.
+extern "C" int ra_sample_traced(const float* logits, int M, int V, const float* temperature,
+                                const int* top_k, const float* top_p, const float* u, int* out, int* path,
+                                void* stream) {
     if (M <= 0) return RA_OK;
     if (V <= 0) return RA_ERR_ARG;
     const size_t lds = (size_t)SAMPLE_BUCKETS * SAMPLE_THREADS * sizeof(float);   // 128 KB: each thread's bins
@@ -251,6 +556,12 @@ extern "C" int ra_sample(const float* logits, int M, int V, const float* tempera
         allowed = true;
     }
     hipLaunchKernelGGL(sample_kernel, dim3(M), dim3(SAMPLE_THREADS), lds, (hipStream_t)stream, logits,
-                       V, temperature, top_k, top_p, u, out);
+                       V, temperature, top_k, top_p, u, out, path);
     return ra_launch_status();
+}
+
+extern "C" int ra_sample(const float* logits, int M, int V, const float* temperature,
+                         const int* top_k, const float* top_p, const float* u, int* out,
+                         void* stream) {
+    return ra_sample_traced(logits, M, V, temperature, top_k, top_p, u, out, nullptr, stream);
 }

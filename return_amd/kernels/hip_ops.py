@@ -78,6 +78,7 @@ def _declare(lib):
         "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "ra_attention_prefill_tile_rows": [I],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
+        "ra_sample_traced": [P, I, I, P, P, P, P, P, P, P],
         "ra_stream_read": [P, L, P, I, P],
     }
     for name, args in sigs.items():
@@ -920,8 +921,10 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------------ sampling
-    def sample(self, logits, temperature, top_k, top_p, u):
-        """Tokens and their raw log-probabilities: int32 [m, 2] (token, float bits of logprob)."""
+    def sample(self, logits, temperature, top_k, top_p, u, path=None):
+        """Tokens and their raw log-probabilities: int32 [m, 2] (token, float bits of logprob).
+        path (int32 [m], optional) is told how each row's thresholds were found: 0 none were needed,
+        1 from the list of the row's largest logits, 2 by passes over the whole row."""
         self._want(logits, "logits", torch.float32, 2)
         M, V = logits.shape
         for t, name, dt in ((temperature, "temperature", torch.float32), (top_k, "top_k", torch.int32),
@@ -930,6 +933,10 @@ class HipOps:
             if t.shape[0] != M:
                 raise KernelError(f"sample: {name} has {t.shape[0]} entries for {M} rows")
         out = torch.empty(M, 2, dtype=torch.int32, device=self.device)
-        self._check(self.lib.ra_sample(_ptr(logits), M, V, _ptr(temperature), _ptr(top_k), _ptr(top_p),
-                                       _ptr(u), _ptr(out), self._stream()), "sample")
+        if path is not None:
+            self._want(path, "path", torch.int32, 1)
+            if path.shape[0] != M:
+                raise KernelError(f"sample: path has {path.shape[0]} entries for {M} rows")
+        self._check(self.lib.ra_sample_traced(_ptr(logits), M, V, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                              _ptr(u), _ptr(out), _ptr(path), self._stream()), "sample")
         return out

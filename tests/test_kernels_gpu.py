@@ -828,10 +828,14 @@ def test_sample_matches_plain_draw(ops, ref, V):
     temp = torch.tensor([0.7, 1.0, 1.3, 0.0] * (M // 4), device=DEV)
     top_k = torch.tensor([0, 5, 0, 3, 50, 0, 1, 0] * (M // 8), dtype=torch.int32, device=DEV)
     top_p = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.3, 0.0, 1.0, 0.95] * (M // 8), device=DEV)
-    a = ops.sample(logits, temp, top_k, top_p, u)
+    path = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+    a = ops.sample(logits, temp, top_k, top_p, u, path=path)
     b = ref.sample(logits, temp, top_k, top_p, u)
     same = (a[:, 0] == b[:, 0]).float().mean().item()
     assert same == 1.0, (a[:, 0].tolist(), b[:, 0].tolist())
+    # a small vocabulary fits the list of the largest logits: every row that needs a threshold takes it from there
+    needs = (temp > 0) & ((top_k > 0) | (top_p < 1))
+    assert torch.equal(path[needs], torch.ones_like(path[needs])) and int(path[~needs].abs().sum()) == 0
     torch.testing.assert_close(a[:, 1].contiguous().view(torch.float32), b[:, 1].contiguous().view(torch.float32),
                                atol=1e-4, rtol=1e-5)
 
@@ -862,6 +866,55 @@ def test_sample_at_the_full_vocabulary(ops):
         assert before - 1e-4 <= float(u[r]) <= float(c[tok]) + 1e-4, (r, tok, before, float(u[r]), float(c[tok]))
         lp = out[r, 1:2].contiguous().view(torch.float32)
         assert abs(float(lp) - plain.chosen_logprob(logits[r].cpu(), tok)) < 1e-3
+
+
+def test_sample_from_the_list_of_the_largest_logits_and_from_the_whole_row(ops):
+    """Rows shaped like a language model's (a bulk of 151,936 logits far below a few hundred large ones)
+    take their thresholds and their token from the list of the largest; rows whose large ones crowd into
+    one wave's run of the row, whose k is more than the list holds, or whose top_p reaches into the bulk
+    go over the whole row. Either way the token is where the plain distribution's running sum, in
+    vocabulary order, passes the row's uniform number."""
+    from tests.plain import qwen3_plain as plain
+    V = 151936
+    g = torch.Generator().manual_seed(21)
+    base = torch.randn(V, generator=g) * 1.5
+    def row(n_large, where, top=12.0):
+        x = base.clone()
+        idx = where[torch.randperm(len(where), generator=g)[:n_large]]
+        x[idx] = 14.0 + 8.0 * torch.rand(n_large, generator=g)          # the large ones: 14 to 22
+        x[idx[0]] = 14.0 + top                                           # and the largest
+        return x
+    everywhere, crowded = torch.arange(V), torch.arange(3000, 9000)
+    cases = [   # logits, temperature, top_k, top_p, path expected
+        (row(300, everywhere), 1.0, 0, 0.9, 1), (row(300, everywhere), 1.0, 40, 1.0, 1),
+        (row(300, everywhere), 0.7, 100, 0.8, 1), (row(2000, everywhere), 1.2, 0, 0.95, 1),
+        (row(2000, everywhere), 1.0, 1500, 0.99, 1), (row(300, everywhere), 1.0, 1, 1.0, 1),
+        (row(300, everywhere), 1.0, 0, 0.01, 1), (row(40, everywhere), 1.0, 0, 0.999, 1),
+        (row(700, crowded), 1.0, 0, 0.9, 2),                 # more than 512 large ones in one wave's run
+        (row(300, everywhere), 1.0, 5000, 1.0, 2),           # k beyond the list
+        (row(1, everywhere, top=9.0), 1.0, 0, 0.999999, 2),  # the list (one token) has less than top_p of the mass: the boundary lies in the bulk
+        (row(3, everywhere, top=3.0), 4.0, 0, 0.9, 2),       # a hot row: the whole vocabulary is within the span
+        (row(300, everywhere), 1.0, 0, 1.0, 0),              # no threshold at all
+    ]
+    M = len(cases)
+    logits = torch.stack([c[0] for c in cases]).to(DEV)
+    temp = torch.tensor([c[1] for c in cases], device=DEV)
+    top_k = torch.tensor([c[2] for c in cases], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([c[3] for c in cases], device=DEV)
+    for seed in (1, 2, 3):
+        u = torch.rand(M, generator=torch.Generator().manual_seed(seed)).to(DEV)
+        path = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+        out = ops.sample(logits, temp, top_k, top_p, u, path=path).cpu()
+        assert path.tolist() == [c[4] for c in cases]
+        for r in range(M):
+            d = plain.sample_distribution(logits[r].cpu(), float(temp[r]), int(top_k[r]), float(top_p[r]))
+            tok = int(out[r, 0])
+            assert d[tok] > 0, f"row {r}: token {tok} is not among the kept ones"
+            c = d.cumsum(0)
+            before = float(c[tok - 1]) if tok else 0.0
+            assert before - 1e-4 <= float(u[r]) <= float(c[tok]) + 1e-4, (r, tok, before, float(u[r]), float(c[tok]))
+            lp = out[r, 1:2].contiguous().view(torch.float32)
+            assert abs(float(lp) - plain.chosen_logprob(logits[r].cpu(), tok)) < 1e-3
 
 
 def test_sample_distribution(ops):
