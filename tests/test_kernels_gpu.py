@@ -819,7 +819,7 @@ def test_sample_greedy_and_logprob(ops, V):
     torch.testing.assert_close(lp.double(), want, atol=1e-4, rtol=1e-5)
 
 
-@pytest.mark.parametrize("V", [97, 1000])
+@pytest.mark.parametrize("V", [97, 1000, 20001])
 def test_sample_matches_plain_draw(ops, ref, V):
     M = 64
     logits = rnd(M, V, seed=72, scale=2.0)
@@ -833,9 +833,11 @@ def test_sample_matches_plain_draw(ops, ref, V):
     b = ref.sample(logits, temp, top_k, top_p, u)
     same = (a[:, 0] == b[:, 0]).float().mean().item()
     assert same == 1.0, (a[:, 0].tolist(), b[:, 0].tolist())
-    # a small vocabulary fits the list of the largest logits: every row that needs a threshold takes it from there
+    # a small vocabulary fits the list of the largest logits: every row that needs a threshold takes it from
+    # there; 20,001 flat logits (an odd number: no 16-byte loads) do not fit, and the search goes over the row
     needs = (temp > 0) & ((top_k > 0) | (top_p < 1))
-    assert torch.equal(path[needs], torch.ones_like(path[needs])) and int(path[~needs].abs().sum()) == 0
+    assert torch.equal(path[needs], torch.full_like(path[needs], 1 if V <= 8192 else 2))
+    assert int(path[~needs].abs().sum()) == 0
     torch.testing.assert_close(a[:, 1].contiguous().view(torch.float32), b[:, 1].contiguous().view(torch.float32),
                                atol=1e-4, rtol=1e-5)
 
