@@ -21,7 +21,6 @@
 #include "common.h"
 
 #define SAMPLE_THREADS 1024
-#define SAMPLE_BUCKETS 32
 #define CAND_WAVES (SAMPLE_THREADS / 64)
 #define CAND_PER_WAVE 512                                        // list entries of one wave's run of the row
 #define CAND_OWN (CAND_WAVES * CAND_PER_WAVE / SAMPLE_THREADS)   // entries a thread looks after in a search: 8
@@ -59,68 +58,83 @@ __device__ __forceinline__ void for_each_logit(const float* __restrict__ x, int 
     }
 }
 
-// One thread's end of a pass of the threshold search: tot[b] is the measure of run b of (lo, hi], cut into
-// nb runs of 2^sh keys. Run b ends at key T_b = lo + ((b + 1) << sh) - 1; the measure above T_b is above_hi
-// plus the runs above b. The threshold lies in the lowest run whose end has at most `limit` above it.
-__device__ __forceinline__ void narrow_range(uint32_t lo, uint32_t hi, int sh, int nb, float above_hi, float limit,
-                                             const float* tot, uint32_t* sh_range, float* sh_above) {
-    float above = above_hi;
-    int b = nb - 1;
-    while (b > 0 && above + tot[b] <= limit) {
-        above += tot[b];
-        --b;
-    }
-    const unsigned long long end = (unsigned long long)lo + (((unsigned long long)b + 1ull) << sh) - 1ull;
-    sh_range[1] = end < (unsigned long long)hi ? (uint32_t)end : hi;
-    sh_range[0] = b == 0 ? lo : lo + ((uint32_t)b << sh);   // the run below ends with more than `limit` above it
-    sh_above[0] = above;
+// Measures are whole numbers: a token counts 2^40 (top-k), or weighs exp((x - gmax) / T) as a multiple of
+// 2^-40 (top-p; what weighs less than 2^-41 of the largest token weighs nothing). Sums of whole numbers do
+// not depend on the order in which they are formed, so they may be formed by atomics, by any number of
+// threads, and come out the same in every run of the program.
+typedef unsigned long long fixed_t;
+#define FIXED_ONE_F 1099511627776.0f               // 2^40
+__device__ __forceinline__ fixed_t to_fixed(float w) {          // 0 <= w <= 1
+    const float t = w * 256.0f;
+    const float hi = floorf(t);
+    return ((fixed_t)(uint32_t)hi << 32) + (fixed_t)(uint32_t)((t - hi) * 4294967296.0f);
 }
 
-// The smallest key t in [lo, hi] with measure{key > t} <= limit, where the measure of a token is 1
-// (MASS false: counts, exact in 32-bit floats below 2^24) or exp((x - gmax) * inv_t) (MASS true), and
-// measure{key > hi} = above_hi <= limit. Every pass over the row cuts [lo, hi] into up to 32 runs of
-// equal width and finds the run that holds t, so that a range of 2^32 keys takes seven passes. A thread
-// adds what its tokens weigh into bins of its own in LDS ([run][thread]); the bins are then added over
-// the threads in a fixed order, so that the result is the same in every run of the program.
-template <bool MASS>
-__device__ uint32_t find_threshold(const float* __restrict__ x, int V, int tid, uint32_t lo, uint32_t hi,
-                                   float above_hi, float limit, float gmax, float inv_t, float* bins, float* part2,
-                                   float* tot, uint32_t* sh_range, float* sh_above) {
+// Sum of whole numbers over the block; every thread gets it. wsum: CAND_WAVES words of LDS.
+__device__ __forceinline__ fixed_t block_sum_fixed(fixed_t v, fixed_t* wsum) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = v;
+    __syncthreads();
+    fixed_t t = 0ull;
+    for (int w = 0; w < CAND_WAVES; ++w) t += wsum[w];
+    __syncthreads();
+    return t;
+}
+
+// The smallest key t in [lo, hi] with measure{key > t} <= limit, given measure{key > hi} = 0. visit(lo, hi, f)
+// calls f(key, measure) for every token with lo < key <= hi that this thread looks after (all threads
+// together: every such token once).
+// A pass cuts (lo, hi] into up to SEARCH_BUCKETS runs of equal width, adds the tokens' measures into the
+// runs (fx, LDS atomics) and finds the highest run b with more than `limit` at and above it: t lies in it.
+// A range of 2^32 keys takes three passes. wsum: CAND_WAVES words, sh_b, sh_above: one word each, all LDS.
+#define SEARCH_BITS 11
+#define SEARCH_BUCKETS (1 << SEARCH_BITS)
+template <typename Visit>
+__device__ uint32_t search_threshold(Visit visit, int tid, uint32_t lo, uint32_t hi, fixed_t limit, fixed_t* fx,
+                                     fixed_t* wsum, int* sh_b, fixed_t* sh_above) {
+    static_assert(SEARCH_BUCKETS == 2 * SAMPLE_THREADS, "a thread looks after two runs");
+    const int wave = tid >> 6, lane = tid & 63;
+    fixed_t above_hi = 0ull;
     while (lo < hi) {
         const uint32_t width = hi - lo;
         const int bits = 32 - __builtin_clz(width);
-        const int sh = bits > 5 ? bits - 5 : 0;                  // (width >> sh) < 32
-        const int nb = (int)(width >> sh) + 1;
+        const int sh = bits > SEARCH_BITS ? bits - SEARCH_BITS : 0;       // (width >> sh) < SEARCH_BUCKETS
+        fx[2 * tid] = 0ull;
+        fx[2 * tid + 1] = 0ull;
+        if (tid == 0) *sh_b = 0;
+        __syncthreads();
+        visit(lo, hi, [&](uint32_t key, fixed_t m) { atomicAdd(&fx[(key - lo) >> sh], m); });
+        __syncthreads();
+        // at_and_above(b) = the measure of runs b and higher; this thread has runs 2 tid and 2 tid + 1
+        const fixed_t f0 = fx[2 * tid], f1 = fx[2 * tid + 1];
+        fixed_t from_here = f0 + f1;                                      // then: over this and the higher threads
 #pragma unroll
-        for (int b = 0; b < SAMPLE_BUCKETS; ++b) bins[b * SAMPLE_THREADS + tid] = 0.f;
-        for_each_logit(x, V, tid, [&](int, float v) {
-            const uint32_t key = order_key(v);
-            if (key > lo && key <= hi) {
-                const float w = MASS ? __expf((v - gmax) * inv_t) : 1.0f;
-                bins[((key - lo) >> sh) * SAMPLE_THREADS + tid] += w;
-            }
-        });
-        __syncthreads();
-        {                                                       // thread (b, j) adds bins[b][j], [j + 32], ...
-            const int b = tid >> 5, j = tid & 31;
-            float t = 0.f;
-#pragma unroll 8
-            for (int i = 0; i < SAMPLE_THREADS / 32; ++i) t += bins[b * SAMPLE_THREADS + j + 32 * i];
-            part2[tid] = t;
+        for (int o = 1; o < 64; o <<= 1) {
+            const fixed_t t = __shfl_down(from_here, o, 64);
+            if (lane + o < 64) from_here += t;
         }
+        if (lane == 0) wsum[wave] = from_here;
         __syncthreads();
-        if (tid < SAMPLE_BUCKETS) {
-            float t = 0.f;
-#pragma unroll 8
-            for (int j = 0; j < 32; ++j) t += part2[tid * 32 + j];
-            tot[tid] = t;
-        }
+        for (int w = wave + 1; w < CAND_WAVES; ++w) from_here += wsum[w];
+        const fixed_t s0 = from_here, s1 = from_here - f0;               // at_and_above(2 tid), (2 tid + 1)
+        // the highest run with more than `limit` at and above it (run 0 if there is none)
+        const int mine = above_hi + s1 > limit ? 2 * tid + 1 : (above_hi + s0 > limit ? 2 * tid : 0);
+        if (mine > 0) atomicMax(sh_b, mine);
         __syncthreads();
-        if (tid == 0) narrow_range(lo, hi, sh, nb, above_hi, limit, tot, sh_range, sh_above);
+        const int b = *sh_b;
+        // what lies above run b: at_and_above(b + 1)
+        if (b + 1 == 2 * tid) *sh_above = above_hi + s0;
+        if (b + 1 == 2 * tid + 1) *sh_above = above_hi + s1;
+        if (b + 1 == SEARCH_BUCKETS && tid == 0) *sh_above = above_hi;
         __syncthreads();
-        lo = sh_range[0];
-        hi = sh_range[1];
-        above_hi = sh_above[0];
+        above_hi = *sh_above;
+        // run b ends at key lo + ((b + 1) << sh) - 1
+        const unsigned long long end = (unsigned long long)lo + (((unsigned long long)b + 1ull) << sh) - 1ull;
+        const uint32_t new_hi = end < (unsigned long long)hi ? (uint32_t)end : hi;
+        lo = b == 0 ? lo : lo + ((uint32_t)b << sh);
+        hi = new_hi;
         __syncthreads();
     }
     return lo;
@@ -156,54 +170,17 @@ __device__ __forceinline__ float wave_running_sum(float v, int lane) {
     return v;
 }
 
-// find_threshold over the list instead of the row: a thread holds CAND_OWN entries (key 0 where the list
-// has none). The measure of a run is added up in whole numbers, a token's weight as a multiple of 2^-40
-// (1 for counts), by LDS atomics: such sums do not depend on the order in which they are formed, so the
-// result is the same in every run of the program. fx: [SAMPLE_BUCKETS] 64-bit words of LDS.
-#define LIST_ONE 1099511627776.0f                  // 2^40
-template <bool MASS>
-__device__ uint32_t list_threshold(const uint32_t (&key)[CAND_OWN], const float (&weight)[CAND_OWN], int tid,
-                                   uint32_t lo, uint32_t hi, float limit, unsigned long long* fx, float* tot,
-                                   uint32_t* sh_range, float* sh_above) {
-    unsigned long long wfx[CAND_OWN];
-#pragma unroll
-    for (int e = 0; e < CAND_OWN; ++e) wfx[e] = MASS ? (unsigned long long)(weight[e] * LIST_ONE + 0.5f) : (1ull << 40);
-    float above_hi = 0.f;
-    while (lo < hi) {
-        const uint32_t width = hi - lo;
-        const int bits = 32 - __builtin_clz(width);
-        const int sh = bits > 5 ? bits - 5 : 0;
-        const int nb = (int)(width >> sh) + 1;
-        if (tid < SAMPLE_BUCKETS) fx[tid] = 0ull;
-        __syncthreads();
-#pragma unroll
-        for (int e = 0; e < CAND_OWN; ++e)
-            if (key[e] > lo && key[e] <= hi) atomicAdd(&fx[(key[e] - lo) >> sh], wfx[e]);
-        __syncthreads();
-        if (tid < SAMPLE_BUCKETS) tot[tid] = (float)fx[tid] * (1.0f / LIST_ONE);
-        __syncthreads();
-        if (tid == 0) narrow_range(lo, hi, sh, nb, above_hi, limit, tot, sh_range, sh_above);
-        __syncthreads();
-        lo = sh_range[0];
-        hi = sh_range[1];
-        above_hi = sh_above[0];
-        __syncthreads();
-    }
-    return lo;
-}
-
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ u,
     int* __restrict__ out, int* __restrict__ path) {
-    extern __shared__ __attribute__((aligned(16))) float bins[];          // [SAMPLE_BUCKETS][SAMPLE_THREADS]
+    extern __shared__ __attribute__((aligned(16))) float dyn[];           // the list (64 KB), then the search's runs (16 KB)
     __shared__ float scratch[16];
-    __shared__ float part[SAMPLE_THREADS];
-    __shared__ float tot[SAMPLE_BUCKETS];
-    __shared__ uint32_t sh_range[2];
     __shared__ float wmass[CAND_WAVES];
-    __shared__ unsigned long long fx[SAMPLE_BUCKETS];
-    __shared__ float sh_f[2];
+    __shared__ fixed_t wsum[CAND_WAVES];
+    __shared__ fixed_t sh_above;
+    __shared__ int sh_b;
+    fixed_t* fx = reinterpret_cast<fixed_t*>(dyn + 2 * CAND_WAVES * CAND_PER_WAVE);
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* x = logits + (size_t)row * V;
 
@@ -286,8 +263,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     if (want_k || want_p) {
         // ---- the list: wave w goes through its run of the row, 64 tokens a load, and appends the tokens
         // within CAND_SPAN of the largest to its part of the list, in their order
-        float* cv = bins;                                                  // [CAND_WAVES][CAND_PER_WAVE] logits
-        int* ci = reinterpret_cast<int*>(bins + CAND_WAVES * CAND_PER_WAVE);   // and their token numbers
+        float* cv = dyn;                                                   // [CAND_WAVES][CAND_PER_WAVE] logits
+        int* ci = reinterpret_cast<int*>(dyn + CAND_WAVES * CAND_PER_WAVE);    // and their token numbers
         __shared__ int cnt[CAND_WAVES];
         __shared__ int sh_over;
         const float cut = gmax - CAND_SPAN * temp;
@@ -345,9 +322,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             bool listed = sh_over == 0 && cut_key > 0u && (!want_k || k <= total);
 
             // a thread's entries for the searches: place (tid % CAND_PER_WAVE) of every other wave's part
-            uint32_t key[CAND_OWN];
-            float weight[CAND_OWN];
             if (listed) {
+                uint32_t key[CAND_OWN];
+                fixed_t weight[CAND_OWN];
                 const int half = tid / CAND_PER_WAVE, off = tid - half * CAND_PER_WAVE;
 #pragma unroll
                 for (int e = 0; e < CAND_OWN; ++e) {
@@ -355,22 +332,33 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                     const bool there = off < cnt[w];
                     const float v = there ? cv[w * CAND_PER_WAVE + off] : 0.f;
                     key[e] = there ? order_key(v) : 0u;
-                    weight[e] = there ? __expf((v - gmax) * inv_t) : 0.f;
+                    weight[e] = there ? to_fixed(__expf((v - gmax) * inv_t)) : 0ull;
                 }
                 // top-k: the k-th largest is on the list; below cut_key - 1 nothing of it lies
                 if (want_k)
-                    keep_key = list_threshold<false>(key, weight, tid, cut_key - 1u, top_key, (float)(k - 1), fx, tot,
-                                                     sh_range, sh_f);
-                if (want_p) {
-                    float zc = 0.f;
+                    keep_key = search_threshold(
+                        [&](uint32_t lo, uint32_t hi, auto add) {
 #pragma unroll
-                    for (int e = 0; e < CAND_OWN; ++e) zc += key[e] >= keep_key && key[e] != 0u ? weight[e] : 0.f;
-                    zc = block_sum(zc, scratch);
-                    const float z = zc + z_rest;
+                            for (int e = 0; e < CAND_OWN; ++e)
+                                if (key[e] > lo && key[e] <= hi) add(key[e], 1ull << 40);
+                        },
+                        tid, cut_key - 1u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above);
+                if (want_p) {
+                    fixed_t zc = 0ull;
+#pragma unroll
+                    for (int e = 0; e < CAND_OWN; ++e) zc += key[e] >= keep_key && key[e] != 0u ? weight[e] : 0ull;
+                    zc = block_sum_fixed(zc, wsum);
+                    const fixed_t z = zc + (fixed_t)((double)z_rest * (double)FIXED_ONE_F);
+                    const fixed_t limit = (fixed_t)((double)p * (double)z);
                     // the boundary is on the list if the list's mass is more than p of the whole (always, after top-k)
-                    if (want_k || zc > p * z) {
-                        const uint32_t lo = want_k ? keep_key : cut_key - 1u;
-                        keep_key = list_threshold<true>(key, weight, tid, lo, top_key, p * z, fx, tot, sh_range, sh_f);
+                    if (want_k || zc > limit) {
+                        keep_key = search_threshold(
+                            [&](uint32_t lo, uint32_t hi, auto add) {
+#pragma unroll
+                                for (int e = 0; e < CAND_OWN; ++e)
+                                    if (key[e] > lo && key[e] <= hi) add(key[e], weight[e]);
+                            },
+                            tid, want_k ? keep_key : cut_key - 1u, top_key, limit, fx, wsum, &sh_b, &sh_above);
                     } else {
                         listed = false;
                     }
@@ -430,17 +418,29 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         // ---- over the whole row. top-k: the key of the k-th largest value is the smallest key with at most
         // k - 1 tokens above it
         if (want_k)
-            keep_key = find_threshold<false>(x, V, tid, 0u, top_key, 0.f, (float)(k - 1), gmax, inv_t, bins, part, tot,
-                                             sh_range, sh_f);
+            keep_key = search_threshold(
+                [&](uint32_t lo, uint32_t hi, auto add) {
+                    for_each_logit(x, V, tid, [&](int, float v) {
+                        const uint32_t key = order_key(v);
+                        if (key > lo && key <= hi) add(key, 1ull << 40);
+                    });
+                },
+                tid, 0u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above);
         // top-p: the smallest key with at most p of the kept mass above it
         if (want_p) {
-            float z = 0.f;
+            fixed_t z = 0ull;
             for_each_logit(x, V, tid, [&](int, float v) {
-                if (order_key(v) >= keep_key) z += __expf((v - gmax) * inv_t);
+                if (order_key(v) >= keep_key) z += to_fixed(__expf((v - gmax) * inv_t));
             });
-            z = block_sum(z, scratch);
-            keep_key = find_threshold<true>(x, V, tid, keep_key, top_key, 0.f, p * z, gmax, inv_t, bins, part, tot,
-                                            sh_range, sh_f);
+            z = block_sum_fixed(z, wsum);
+            keep_key = search_threshold(
+                [&](uint32_t lo, uint32_t hi, auto add) {
+                    for_each_logit(x, V, tid, [&](int, float v) {
+                        const uint32_t key = order_key(v);
+                        if (key > lo && key <= hi) add(key, to_fixed(__expf((v - gmax) * inv_t)));
+                    });
+                },
+                tid, keep_key, top_key, (fixed_t)((double)p * (double)z), fx, wsum, &sh_b, &sh_above);
         }
     }
 
@@ -547,7 +547,7 @@ extern "C" int ra_sample_traced(const float* logits, int M, int V, const float* 
                                 void* stream) {
     if (M <= 0) return RA_OK;
     if (V <= 0) return RA_ERR_ARG;
-    const size_t lds = (size_t)SAMPLE_BUCKETS * SAMPLE_THREADS * sizeof(float);   // 128 KB: each thread's bins
+    const size_t lds = (size_t)2 * CAND_WAVES * CAND_PER_WAVE * sizeof(float) + SEARCH_BUCKETS * sizeof(fixed_t);   // 80 KB
     static bool allowed = false;
     if (!allowed) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(sample_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
