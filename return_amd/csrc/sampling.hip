@@ -277,6 +277,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             float rest = 0.f;
             const unsigned long long below = (1ull << lane) - 1ull;        // the lanes before this one
             for (int i0 = beg + 4 * lane; i0 - 4 * lane < end; i0 += 4 * 256) {      // four loads on their way
+                if (have > CAND_PER_WAVE) break;          // (a flat row: this run alone is too much for the list)
                 float v[4][4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) load4(i0 + 256 * j, v[j]);
