@@ -788,10 +788,14 @@ def test_decode_attention_that_prepares_q_k_v_itself(ops, monkeypatch, D, Hq, Hk
     assert not ops.attention_qkv(qkv[:4], got[:4], k2, v2, mixed, 0, 1.0, 0, Hq, Hkv, D, wq, wk, 1e-5, cos, sin, R)
 
 
+@pytest.mark.parametrize("split", [0, 64, 256, 1024])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attention_over_a_long_context(ops, ref, dtype):
+def test_attention_over_a_long_context(ops, ref, monkeypatch, dtype, split):
     """40,000 keys in scattered pages: a decoded token at the end of them, one after five keys, and
-    a portion of 300 query rows whose first row sees 39,700 keys; in one step."""
+    a portion of 300 query rows whose first row sees 39,700 keys; in one step. With splits of the
+    decode kernel's own choice and of 64, 256 and 1,024 keys (625, 157 and 40 splits, which the merge
+    takes in eight, eight and four groups of threads)."""
+    monkeypatch.setattr(ops, "decode_split_tokens", split)
     Hq, Hkv, D, P = 8, 2, 128, 16
     segs = [(1, 39_999), (1, 5), (300, 39_700)]
     need = [-(-(a + b) // P) for a, b in segs]
