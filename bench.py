@@ -400,10 +400,34 @@ def contexts_8b(args):
                               "frac": round(prefill_flops(cfg, n) / pf / PEAK_FLOPS[args.dtype], 4)}}
 
 
+def products_8b(args):
+    """The products of a 2,048-token prefill on the Qwen3-8B shape, one by one: the library's product
+    (what the engine uses at these row counts) beside the hand-written tiled MFMA product that stands in
+    where the library cannot be used. Weights of a shape are taken in turn, operands are random."""
+    import torch
+    from return_amd.kernels.hip_ops import HipOps
+    ops = HipOps("cuda:0")
+    torch.manual_seed(0)
+    rows = 2048
+    out = {}
+    for name, N, K in (("qkv", 6144, 4096), ("o", 4096, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)):
+        ws = [(torch.randn(N, K, device="cuda:0") * 0.02).to(torch.bfloat16) for _ in range(4)]
+        x = torch.randn(rows, K, device="cuda:0").to(torch.bfloat16)
+        flops = 2.0 * rows * N * K
+        got = {}
+        for how in ("library", "mfma"):
+            secs = ops._time_over(lambda w, how=how: ops._linear_by(how, x, w, torch.bfloat16), ws, 8)
+            got[how] = {"us": round(secs * 1e6, 1), "TFLOPs": round(flops / secs / 1e12, 1)}
+        out[name] = got
+        del ws
+    return {"metric": "products of a 2,048-token prefill, library and hand-written (Qwen3-8B shape)", "unit": "TFLOP/s",
+            "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "rows": rows, "products": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="decode_8b",
-                    choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b"],
+                    choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -431,7 +455,7 @@ def main():
         return 1
     if args.workload != "decode_8b":
         print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
-                          "contexts_8b": contexts_8b}[args.workload](args)))
+                          "contexts_8b": contexts_8b, "products_8b": products_8b}[args.workload](args)))
         return 0
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),

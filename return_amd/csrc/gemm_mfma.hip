@@ -111,10 +111,19 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16* __restrict__
     }
 }
 
+extern "C" int ra_gemm_tile_bf16(const void* X, const void* W, void* C, int M, int N, int K, int splits,
+                                 int out_dtype, void* stream);
+
+// More than 128 rows go to the product with tiles of 256 x 256 (gemm_tile.hip) where it takes the sizes
+// and has at least 160 tiles to spread over the CUs (2,048 x 4,096 are 128 tiles: there the small tiles
+// are as fast or faster).
 extern "C" int ra_gemm_mfma_bf16(const void* A, const void* W, void* C, int M, int N, int K,
                                  int out_dtype, void* stream) {
     if (M <= 0 || N <= 0) return RA_OK;
     if (K <= 0 || K % 8 != 0) return RA_ERR_ARG;
+    if (M > GM_BM && K % 32 == 0 && (size_t)M * K * 2 <= 0x7fffffffull && (size_t)N * K * 2 <= 0x7fffffffull &&
+        (long long)((M + 255) / 256) * ((N + 255) / 256) >= 160)
+        return ra_gemm_tile_bf16(A, W, C, M, N, K, 1, out_dtype, stream);
     dim3 grid((N + GM_BN - 1) / GM_BN, (M + GM_BM - 1) / GM_BM), block(256);
     if (grid.y > 65535) return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;

@@ -495,9 +495,14 @@ def test_products_for_the_residual_stream_are_measured_at_some_hundred_rows_too(
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,N,K", [(65, 331, 120), (128, 128, 32), (129, 257, 264), (300, 1000, 512), (70, 48, 8)])
+@pytest.mark.parametrize("M,N,K", [(65, 331, 120), (128, 128, 32), (129, 257, 264), (300, 1000, 512), (70, 48, 8),
+                                   (3000, 4300, 32), (2700, 5130, 64), (5130, 2700, 96), (2570, 5000, 160),
+                                   (1290, 10001, 224), (3000, 4500, 256), (4000, 3333, 352), (2048, 6400, 4096)])
 def test_tiled_mfma_product(ops, out_dtype, M, N, K):
-    """The hand-written tiled product for many rows, edges in every dimension."""
+    """The hand-written tiled products for many rows, edges in every dimension: tiles of 128 x 128 up
+    to 128 rows, when K is no multiple of 32 or when larger tiles would be fewer than 160, tiles of 256 x 256
+    otherwise, with 1, 2, 3, 5, 7, 8, 11
+    and 128 k-steps of 32 (the copies run three stages ahead; the loop's steady part starts at seven)."""
     x = rnd(M, K, dtype=torch.bfloat16, seed=47)
     w = rnd(N, K, dtype=torch.bfloat16, seed=48, scale=0.1)
     ops.own_gemm = True
