@@ -852,8 +852,8 @@ def test_sample_matches_plain_draw(ops, ref, V):
 
 
 def test_sample_at_the_full_vocabulary(ops):
-    """top-k and top-p at a vocabulary of 151,936 (the threshold search over seven passes and its
-    bins): every row's token is where the plain distribution's running sum, in vocabulary order,
+    """top-k and top-p at a vocabulary of 151,936 (the threshold search over the whole row, pass by
+    pass): every row's token is where the plain distribution's running sum, in vocabulary order,
     passes the row's uniform number; peaked and flat rows, ties above the boundary (tokens that tie
     with the boundary value itself are all kept here, one by one in the plain rule), k = 1, p near 0."""
     from tests.plain import qwen3_plain as plain
