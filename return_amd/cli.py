@@ -59,7 +59,8 @@ def cmd_generate(args) -> int:
     engine = Engine(args.model, max_token=args.max_token, max_reside=args.max_reside, dtype=args.dtype,
                     page_size=args.page_size, seed=args.seed, max_step_tokens=args.max_step_tokens,
                     prefill_chunk=args.prefill_chunk, use_graphs=not args.no_graphs,
-                    tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
+                    tune_products=not args.no_tune, defer_norms=not args.no_defer_norms,
+                    check_invariants=args.check_invariants)
     # Requests are run together until a session_id comes again: that request is a later turn of the
     # session (the reference keeps a session's cache for its next request, rollout/engine.py:286-306,
     # which sends the whole conversation again, 266-274). A session's cache is kept while more of
@@ -124,6 +125,8 @@ def main(argv=None) -> int:
                    help="run every RMSNorm as a kernel of its own instead of inside the products around it")
     g.add_argument("--no-tune", action="store_true",
                    help="choose the kernel of every projection by rule instead of measuring at load")
+    g.add_argument("--check-invariants", action="store_true",
+                   help="debugging: check after every step that no cache page or slot is lost or held twice")
     g.add_argument("--requests", help="file of JSON lines (or - for standard input), one request each")
     g.add_argument("--prompt-ids", help="one prompt as comma-separated token ids")
     g.add_argument("--max-new-tokens", type=int, default=32)

@@ -22,6 +22,9 @@ class EngineConfig:
     lookahead: bool = True             # launch every step before the sampled tokens of the one before it are read
     tune_products: bool = True         # measure at load which kernel forms each projection fastest at few rows
     defer_norms: bool = True           # steps of few rows: finish every RMSNorm inside the products around it (two kernels less per layer)
+    check_invariants: bool = False     # debugging: after every step and every freed request the cache manager checks that no page
+                                       # or slot is lost, held twice, or both free and held (the reference's audit wraps its cache's
+                                       # methods the same way, rollout/utils/check_search_swap_timing.py:107-138)
     seed: int = 0                      # base seed of the sampling streams
     device: str = "cuda:0"
 

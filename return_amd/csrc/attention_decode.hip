@@ -560,7 +560,10 @@ extern "C" int ra_dec_part_3(DEC_PART_ARGS);
 // The kernel is a chain of loads that wait for each other (the request's tables, then the splits'
 // maxima, then their sums), and each link costs about a microsecond after a kernel that wrote them.
 // So a thread's COMBINE_AHEAD splits' maxima and sums are asked for at once with the tables, before it
-// is known how many splits hold keys: what a split beyond them left in memory is read and not used.
+// is known how many splits hold keys: what a split beyond them left in memory (never written by this
+// call: whatever the allocator, or an earlier call on the library's own buffer, left there) is read,
+// at addresses clamped to the request's max_splits places, and not used: every use below is guarded
+// by s < ns, and that guard must stay ahead of the arithmetic, since such values may be NaN.
 // A request of more than COMBINE_AHEAD splits has GROUPS groups of 128 threads, each for a run of
 // at most COMBINE_AHEAD consecutive splits (or more, by a loop, beyond 8 groups' worth), so that all
 // loads of a long request are on their way together; the groups' sums are merged through LDS in group

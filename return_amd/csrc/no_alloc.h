@@ -1,9 +1,8 @@
 // The one entry point of the library that allocates nothing.
 //
-// It has no counterpart in the reference (whose decode attention gets its partial sums from
-// torch's allocator, rollout/attention.py:543-599). It is for callers that cannot allocate
-// device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
-// hipMalloc. Every other entry point takes the memory for partial results from its caller.
+// It has no counterpart in the reference. It is for callers that cannot allocate device
+// memory: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+// Every other entry point takes the memory for partial results from its caller.
 #pragma once
 
 #ifdef __cplusplus
@@ -22,7 +21,11 @@ extern "C" {
 // on the device that is current at the call (the stream must belong to it). Beyond
 // RA_DECODE_STATIC_FLOATS the call is refused with RA_ERR_SCRATCH and nothing is launched.
 // No hipMalloc, hipFree or other allocating routine is called. Nothing in the buffer has to start
-// at zero: every split that the merge reads has been written by the same call. All calls on one
+// at zero: every split whose values the merge uses has been written by the same call. (The merge
+// kernel asks for a fixed number of splits' sums before it knows how many of them hold keys; what
+// an earlier call, or nobody, left in the places of the others is loaded, within the buffer, and
+// discarded by the test `s < ns` before any arithmetic. That test must stay ahead of the sums.)
+// All calls on one
 // GPU share that GPU's buffer, so two calls that overlap in time on one GPU (different streams,
 // threads or processes' graphs on the same library instance) race; calls on one stream do not.
 // With merge != 0 the splits are merged inside the workgroups and the buffer is not touched.

@@ -218,6 +218,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         if (wm[w] > gmax) { gmax = wm[w]; argmax = wa[w]; }
         else if (wm[w] == gmax) argmax = min(argmax, wa[w]);
     }
+    // a row with no value above -inf (all -inf, or NaN after an overflow upstream) never set an index:
+    // token 0 then, so that nothing below reads beyond the row
+    if ((unsigned)argmax >= (unsigned)V) argmax = 0;
     float total_e = 0.f;
     for (int w = 0; w < SAMPLE_THREADS / 64; ++w)
         total_e += (wm[w] == -INFINITY) ? 0.f : ws[w] * __expf(wm[w] - gmax);

@@ -67,6 +67,9 @@ class StepBatch:
     # q tiles of the prefill attention kernel, by rows per tile: rows -> int32 [tiles, 2] of
     # (request number, first row of the tile among the request's new tokens)
     prefill_tiles: dict = dataclasses.field(default_factory=dict)
+    # further integers per token that a part of the model asked for (step_needs()["token_columns"]), by name:
+    # int32 [T] each; what a request does not bring for its tokens is their position
+    token_columns: dict = dataclasses.field(default_factory=dict)
 
 
 
@@ -82,11 +85,15 @@ def prefill_tiles(q_lens, q_starts=None, rows=64):
 class StepBuilder:
     """Fixed device buffers for the tables of a step, sized for the worst case."""
 
-    def __init__(self, cache: CacheManager, max_step_tokens: int, max_requests: int, device, tile_rows=()):
+    def __init__(self, cache: CacheManager, max_step_tokens: int, max_requests: int, device, tile_rows=(),
+                 token_columns=()):
         """tile_rows: heights of the q tiles that the model's mixers want listed for the requests that
-        bring more than one token (what their attention kernels' grids run over); none: no lists."""
+        bring more than one token (what their attention kernels' grids run over); none: no lists.
+        token_columns: names of further integers per token that parts of the model read beside the
+        position (a position encoding with more than one axis, say)."""
         self.cache = cache
         self.tile_rows = tuple(sorted(int(r) for r in tile_rows))
+        self.token_columns = tuple(sorted(str(c) for c in token_columns))
         self.device = torch.device(device)
         self.max_tokens = int(max_step_tokens)
         self.max_requests = int(max_requests)
@@ -95,6 +102,7 @@ class StepBuilder:
                   ("q_start", N), ("seq_lens", N), ("slot_ids", N), ("decode_segs", N),
                   ("prefill_toks", T)]
         layout += [(f"prefill_tiles{rows}", 2 * (T // rows + N)) for rows in self.tile_rows]
+        layout += [(f"column_{name}", T) for name in self.token_columns]
         for g in range(G):
             layout += [(f"slot_mapping{g}", T), (f"cu_pages{g}", N + 1), (f"kv_start{g}", N)]
         self._small_end = None
@@ -136,8 +144,10 @@ class StepBuilder:
         return self._dev[off:off + k]
 
     def build(self, tables: StepTables, tokens: Sequence[Sequence[int]],
-              logit_rows: Sequence[int]) -> StepBatch:
-        """tokens[i] are the new tokens of request i; logit_rows index the step's flat token rows."""
+              logit_rows: Sequence[int], columns: Optional[dict] = None) -> StepBatch:
+        """tokens[i] are the new tokens of request i; logit_rows index the step's flat token rows;
+        columns: name -> T integers for the token columns the builder was made with (a name that is
+        missing gets the tokens' positions)."""
         n = len(tables.request_ids)
         T = int(tables.cu_q[-1])
         if T > self.max_tokens:
@@ -152,6 +162,16 @@ class StepBuilder:
             raise ValueError("tokens do not match the step's q_lens")
         self._put("token_ids", flat)
         self._put("positions", tables.positions)
+        for name in self.token_columns:
+            col = (columns or {}).get(name)
+            col = tables.positions if col is None else np.asarray(col, dtype=np.int32)
+            if len(col) != T:
+                raise ValueError(f"token column {name!r} has {len(col)} entries for {T} tokens")
+            self._put(f"column_{name}", col)
+        unknown = set(columns or ()) - set(self.token_columns)
+        if unknown:
+            raise ValueError(f"token column(s) {sorted(unknown)} are not among those the model reads: "
+                             f"{list(self.token_columns)}")
         m = self._put("logit_rows", np.asarray(logit_rows, dtype=np.int32))
         self._put("cu_q", tables.cu_q)
         self._put("q_start", tables.q_start)
@@ -214,4 +234,5 @@ class StepBuilder:
             prefill_toks=self._view("prefill_toks", n_pre_tok) if mixed_kinds else None,
             prefill_segs=pre,
             prefill_tiles={rows: self._view(f"prefill_tiles{rows}", 2 * len(t)).view(-1, 2)
-                           for rows, t in tiles.items()})
+                           for rows, t in tiles.items()},
+            token_columns={name: self._view(f"column_{name}", T) for name in self.token_columns})

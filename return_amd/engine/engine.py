@@ -69,16 +69,22 @@ class Engine:
 
     # ------------------------------------------------------------------ requests
     def submit(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
-               request_id=None, keep: bool = False) -> Request:
+               request_id=None, keep: bool = False, token_columns=None) -> Request:
         """Queue a request. request_id names its session (the reference's session_id,
         rollout/server.py:25-42); with keep, what the cache holds when it ends stays under that id,
         and a later request with the same id whose prompt repeats those tokens and goes on computes
-        only the rest (rollout/engine.py:266-274, 286-306). release() gives a kept session back."""
+        only the rest (rollout/engine.py:266-274, 286-306). release() gives a kept session back.
+        token_columns: name -> one integer per prompt token, for a model whose parts read further
+        integers per token beside the position (see Request)."""
         params = params or SamplingParams()
         self.check_prompt(prompt_ids)
         n = self._submitted
         self._submitted += 1
-        r = Request(request_id if request_id is not None else n, prompt_ids, params, keep=keep)
+        unknown = set(token_columns or ()) - set(self.runner.builder.token_columns)
+        if unknown:
+            raise ValueError(f"token column(s) {sorted(unknown)}: the model reads {list(self.runner.builder.token_columns)}")
+        r = Request(request_id if request_id is not None else n, prompt_ids, params, keep=keep,
+                    token_columns=token_columns)
         r.stream = UniformStream(self.config.seed, params.seed if params.seed is not None else n)
         self.scheduler.add(r)
         return r
@@ -112,11 +118,14 @@ class Engine:
             # one token each (decoded tokens, or prompts of one token), all known or all still on the
             # device: one call that runs the model and the sampler (from a graph if enabled)
             ids = [e.request.id for e in plan.entries]
+            columns = [e.request.columns_at(e.start, 1) for e in plan.entries]
+            columns = columns if any(columns) else None
             if all(unknown):
-                return self.runner.decode_launch(ids, None, *options, feed_rows=[row_of[i] for i in ids])
-            return self.runner.decode_launch(ids, [e.tokens[0] for e in plan.entries], *options)
-        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [])
-                   for e in plan.entries]
+                return self.runner.decode_launch(ids, None, *options, feed_rows=[row_of[i] for i in ids],
+                                                 columns=columns)
+            return self.runner.decode_launch(ids, [e.tokens[0] for e in plan.entries], *options, columns=columns)
+        entries = [StepEntry(e.request.id, e.tokens, [len(e.tokens) - 1] if e.sample else [],
+                             e.request.columns_at(e.start, len(e.tokens))) for e in plan.entries]
         feed = [(i, row_of[e.request.id]) for i, e in enumerate(plan.entries) if e.tokens[0] is None]
         return self.runner.step_launch(entries, *options, feed=feed)
 
@@ -188,7 +197,8 @@ class Engine:
         try:
             if any(e.sample for e in plan.entries):
                 return self._launch(plan, previous)
-            self.runner.step([StepEntry(e.request.id, e.tokens, []) for e in plan.entries])
+            self.runner.step([StepEntry(e.request.id, e.tokens, [], e.request.columns_at(e.start, len(e.tokens)))
+                              for e in plan.entries])
             return None
         except Exception as error:
             for e in plan.entries:
@@ -199,10 +209,12 @@ class Engine:
     # ------------------------------------------------------------------ whole jobs
     def generate(self, prompts: Sequence[Sequence[int]],
                  params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
-                 session_ids: Optional[Sequence] = None, keep: bool = False) -> List[GenerationResult]:
+                 session_ids: Optional[Sequence] = None, keep: bool = False,
+                 token_columns: Optional[Sequence] = None) -> List[GenerationResult]:
         """Generate for every prompt (lists of token ids); results come in the prompts' order.
         session_ids name the requests (distinct within one call); with keep their caches stay
-        for a later call that goes on with the same sessions."""
+        for a later call that goes on with the same sessions. token_columns: per prompt, what
+        submit() takes under that name (or None)."""
         if params is None or isinstance(params, SamplingParams):
             params = [params or SamplingParams()] * len(prompts)
         if len(params) != len(prompts):
@@ -211,7 +223,10 @@ class Engine:
             raise ValueError("session_ids must name every prompt, each differently")
         for i, p in enumerate(prompts):               # all of them before any is queued
             self.check_prompt(p, f"prompt {i}")
-        requests = [self.submit(p, sp, request_id=None if session_ids is None else session_ids[i], keep=keep)
+        if token_columns is not None and len(token_columns) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but token columns for {len(token_columns)}")
+        requests = [self.submit(p, sp, request_id=None if session_ids is None else session_ids[i], keep=keep,
+                                token_columns=None if token_columns is None else token_columns[i])
                     for i, (p, sp) in enumerate(zip(prompts, params))]
         while self.scheduler.has_work() or self._in_flight is not None:
             before = (self.steps, len(self.scheduler.waiting), len(self.scheduler.running))

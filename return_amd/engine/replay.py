@@ -67,7 +67,8 @@ def main(argv=None) -> int:
         for e in rec.get("entries", []):
             if not runner.is_live(e["id"]):
                 runner.add_request(e["id"])
-            entries.append(StepEntry(e["id"], e["tokens"], e.get("want", [])))
+            # ("columns", name -> one integer per token, only for a model whose parts read such columns)
+            entries.append(StepEntry(e["id"], e["tokens"], e.get("want", []), e.get("columns")))
         logits = runner.step(entries) if entries else None
         if logits is not None and logits.shape[0] > 0:
             arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)

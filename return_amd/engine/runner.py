@@ -26,13 +26,16 @@ from .batch import StepBatch, StepBuilder
 
 
 class StepEntry:
-    """One request's share of a step: its next tokens and the places (among them) whose logits are wanted."""
-    __slots__ = ("request_id", "tokens", "want")
+    """One request's share of a step: its next tokens and the places (among them) whose logits are wanted.
+    columns: name -> one integer per token, for the token columns that parts of the model read beside
+    the position (Decoder.step_needs()["token_columns"]); a column that is not given is the position."""
+    __slots__ = ("request_id", "tokens", "want", "columns")
 
-    def __init__(self, request_id, tokens: Sequence[int], want: Sequence[int] = ()):
+    def __init__(self, request_id, tokens: Sequence[int], want: Sequence[int] = (), columns: Optional[dict] = None):
         self.request_id = request_id
         self.tokens = list(tokens)
         self.want = list(want)
+        self.columns = columns
 
 
 class ModelRunner:
@@ -66,8 +69,9 @@ class ModelRunner:
         self._check_cache_fits()
         self.cache = CacheManager(self.model.cache_layers(), ec.page_size, ec.max_token,
                                   ec.max_reside, self.rt.dtype, self.rt.device)
+        needs = self.model.step_needs()
         self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device,
-                                   tile_rows=self.model.step_needs()["prefill_tile_rows"])
+                                   tile_rows=needs["prefill_tile_rows"], token_columns=needs["token_columns"])
         self.vocab_size = self.spec.vocab_size
         self.max_position = self.spec.max_position
         # decode-only steps replayed from captured HIP graphs (rollout/model.py:346-407 captures one
@@ -115,9 +119,35 @@ class ModelRunner:
 
     def free_request(self, request_id) -> None:
         self.cache.free_request(request_id)
+        if self.engine_config.check_invariants:
+            self.cache.check_invariants()
+
+    def _end_step(self) -> None:
+        self.cache.end_step()
+        if self.engine_config.check_invariants:
+            self.cache.check_invariants()
 
     def is_live(self, request_id) -> bool:
         return request_id in self.cache.live
+
+    def _flat_columns(self, per_entry, tables):
+        """name -> the step's T integers of every token column the model reads, from what the entries
+        bring (per_entry[i]: name -> one integer per token of entry i, or None); the rest are positions.
+        None when no entry brings any."""
+        if not any(per_entry):
+            return None
+        out = {}
+        for i, cols in enumerate(per_entry):
+            for name, values in (cols or {}).items():
+                if name not in self.builder.token_columns:
+                    raise ValueError(f"request {tables.request_ids[i]!r} brings token column {name!r}; the model "
+                                     f"reads {list(self.builder.token_columns)}")
+                a, b = int(tables.cu_q[i]), int(tables.cu_q[i + 1])
+                if len(values) != b - a:
+                    raise ValueError(f"request {tables.request_ids[i]!r}: token column {name!r} has {len(values)} "
+                                     f"entries for {b - a} tokens")
+                out.setdefault(name, tables.positions.copy())[a:b] = values
+        return out
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -153,13 +183,14 @@ class ModelRunner:
             at += n
         tables = self.cache.begin_step([(e.request_id, len(e.tokens)) for e in entries])
         try:
-            batch = self.builder.build(tables, [[0 if t is None else t for t in e.tokens] for e in entries], rows)
+            batch = self.builder.build(tables, [[0 if t is None else t for t in e.tokens] for e in entries], rows,
+                                       self._flat_columns([e.columns for e in entries], tables))
             if after_build is not None:
                 after_build(batch)
             with torch.no_grad():
                 logits = self.model.forward(batch, self.cache)
         finally:
-            self.cache.end_step()
+            self._end_step()
         return logits, batch
 
     def step_launch(self, entries: Sequence[StepEntry], temperature, top_k, top_p, uniforms, feed=None):
@@ -233,7 +264,8 @@ class ModelRunner:
                                     self._samp_dev_f[1, :m], self._samp_dev_f[2, :m])
         return logits, picked
 
-    def decode_launch(self, request_ids, tokens, temperature, top_k, top_p, uniforms, feed_rows=None):
+    def decode_launch(self, request_ids, tokens, temperature, top_k, top_p, uniforms, feed_rows=None,
+                      columns=None):
         """Start one decode step (one token per request, logits sampled at once) and return a
         ticket for decode_collect. Nothing here waits for the device.
 
@@ -242,8 +274,11 @@ class ModelRunner:
         this step can be launched before the previous one's tokens have been read.
         With use_graphs the whole step (model and sampler) is one captured HIP graph per
         (batch size, context bucket); tables and sampling options go into fixed buffers first.
+        columns: per request, name -> [integer] for the token columns the model reads (or None).
         """
         n = len(request_ids)
+        if n == 0:
+            raise ValueError("decode_launch: a decode step needs at least one request")
         if tokens is None:
             if self._last_picked is None or feed_rows is None or len(feed_rows) != n:
                 raise ValueError("decode_launch without tokens needs a previous launch and its rows to take them from")
@@ -267,7 +302,8 @@ class ModelRunner:
         try:
             tables = self.cache.pad_tables(tables, pad)
             host_tokens = [[0]] * rows if tokens is None else [[int(t)] for t in tokens] + [[0]] * pad
-            batch = self.builder.build(tables, host_tokens, list(range(rows)))
+            batch = self.builder.build(tables, host_tokens, list(range(rows)),
+                                       self._flat_columns(list(columns) + [None] * pad, tables) if columns else None)
             if tokens is None:
                 # after the tables' copy and before the step: the sampled tokens become the new tokens
                 if self._samp_copied is not None:
@@ -284,7 +320,7 @@ class ModelRunner:
                 else:
                     logits, picked = self._decode_body(batch)
         finally:
-            self.cache.end_step()
+            self._end_step()
         return self._ticket(picked, n, logits)
 
     def decode_collect(self, ticket):
@@ -345,7 +381,7 @@ class ModelRunner:
                 with torch.cuda.graph(graph, pool=self._graph_pool):
                     logits, picked = self._decode_body(batch)
         finally:
-            self.cache.end_step()
+            self._end_step()
         self._graphs[key] = (graph, logits, picked)
 
     def _replay(self, key):

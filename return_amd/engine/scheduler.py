@@ -29,9 +29,17 @@ class Request:
     """One generation request (the reference's Request, rollout/engine.py:13-62, without paragraphs)."""
 
     def __init__(self, request_id, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
-                 keep: bool = False):
+                 keep: bool = False, token_columns: Optional[Dict[str, Sequence[int]]] = None):
+        """token_columns: name -> one integer per prompt token, for models whose parts read further
+        integers per token beside the position (positions along a second axis, say). Tokens beyond
+        what a column lists (the generated ones) go on counting from its last value."""
         if len(prompt_ids) == 0:
             raise ValueError(f"request {request_id!r} has an empty prompt")
+        self.token_columns = {k: [int(x) for x in v] for k, v in (token_columns or {}).items()}
+        for name, col in self.token_columns.items():
+            if not 0 < len(col) <= len(prompt_ids):
+                raise ValueError(f"request {request_id!r}: token column {name!r} lists {len(col)} values for "
+                                 f"{len(prompt_ids)} prompt tokens")
         self.id = request_id
         self.keep = bool(keep)              # what the cache holds stays under this id when the request ends
         self.resumed = 0                    # tokens of the prompt that were found in the cache at admission
@@ -54,12 +62,23 @@ class Request:
     def finished(self) -> bool:
         return self.status in ("finished", "failed")
 
+    def columns_at(self, start: int, n: int) -> Optional[Dict[str, List[int]]]:
+        """The request's token columns for its tokens start .. start + n - 1, or None if it brings none."""
+        if not self.token_columns:
+            return None
+        out = {}
+        for name, col in self.token_columns.items():
+            k = len(col)
+            out[name] = [col[i] if i < k else col[-1] + (i - k + 1) for i in range(start, start + n)]
+        return out
+
 
 @dataclasses.dataclass
 class PlannedEntry:
     request: Request
     tokens: List[int]
     sample: bool            # the portion reaches the request's last token: its logits are sampled
+    start: int = 0          # place of the first of these tokens in the request's sequence
 
 
 @dataclasses.dataclass
@@ -229,7 +248,8 @@ class Scheduler:
             n = min(n_prompt - computed, self.prefill_chunk, budget)
             if n <= 0:
                 return
-            entries.append(PlannedEntry(r, r.prompt_ids[computed:computed + n], sample=(computed + n == n_prompt)))
+            entries.append(PlannedEntry(r, r.prompt_ids[computed:computed + n], sample=(computed + n == n_prompt),
+                                        start=computed))
             budget -= n
 
         for r in self.running:                      # decoding requests first
@@ -239,9 +259,9 @@ class Scheduler:
             if e is not None and e.sample:
                 if outputs >= r.max_new:            # the step under way brings its last token
                     continue
-                entries.append(PlannedEntry(r, [None], sample=True))
+                entries.append(PlannedEntry(r, [None], sample=True, start=computed))
             else:
-                entries.append(PlannedEntry(r, [r.output[-1]], sample=True))
+                entries.append(PlannedEntry(r, [r.output[-1]], sample=True, start=computed))
             budget -= 1
         for r in self.running:                      # prompts under way
             computed, _, _ = state(r)

@@ -63,13 +63,20 @@ class Decoder:
             spec = self.blocks[call.block].cache_spec()
             if spec is None:
                 raise ValueError(f"block {call.block} keeps nothing but the run order gives it cache layer {call.cache}")
-            if call.cache in need and need[call.cache] != spec:
-                raise ValueError(f"cache layer {call.cache} is used by mixers with different needs")
-            need[call.cache] = spec
-            if call.writes_cache:
-                if call.cache in writers:
-                    raise ValueError(f"cache layer {call.cache} has two writers in the run order")
-                writers.add(call.cache)
+            # a block that keeps several things names them as a tuple, and the call a cache layer for each
+            specs = tuple(spec) if isinstance(spec, (tuple, list)) else (spec,)
+            layers = tuple(call.cache) if isinstance(call.cache, (tuple, list)) else (call.cache,)
+            if len(specs) != len(layers):
+                raise ValueError(f"block {call.block} keeps {len(specs)} things but the run order gives it "
+                                 f"cache layers {call.cache}")
+            for layer, one in zip(layers, specs):
+                if layer in need and need[layer] != one:
+                    raise ValueError(f"cache layer {layer} is used by mixers with different needs")
+                need[layer] = one
+                if call.writes_cache:
+                    if layer in writers:
+                        raise ValueError(f"cache layer {layer} has two writers in the run order")
+                    writers.add(layer)
         missing = set(need) - writers
         if missing:
             raise ValueError(f"cache layers {sorted(missing)} are read but never written")
@@ -77,19 +84,25 @@ class Decoder:
 
     def step_needs(self):
         """What the parts ask of a step's tables beyond what every step has, merged over the model:
-        {"prefill_tile_rows": set of q-tile heights whose tile lists the attention kernels read}."""
-        tile_rows = set()
-        for block in self.blocks:
-            needs = block.step_needs() if hasattr(block, "step_needs") else {}
+        {"prefill_tile_rows": set of q-tile heights whose tile lists the attention kernels read,
+         "token_columns": set of names of further integers per token (StepBatch.token_columns) that a
+         block, a position encoding or the embedding reads beside the position}."""
+        tile_rows, columns = set(), set()
+        for part in list(self.blocks) + list(self.positions.values()) + [self.embedding]:
+            needs = part.step_needs() if hasattr(part, "step_needs") else {}
             tile_rows.update(needs.get("prefill_tile_rows", ()))
-        return {"prefill_tile_rows": tile_rows}
+            columns.update(needs.get("token_columns", ()))
+        return {"prefill_tile_rows": tile_rows, "token_columns": columns}
 
     def forward(self, step, cache):
         """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
         h = self.embedding.forward(step.token_ids, step)
         pending = None
         for i, call in enumerate(self.schedule):
-            view = cache.view(call.cache) if call.cache is not None else None
+            view = None
+            if call.cache is not None:
+                view = tuple(cache.view(c) for c in call.cache) if isinstance(call.cache, (tuple, list)) \
+                    else cache.view(call.cache)
             block = self.blocks[call.block]
             if getattr(block, "first_norm", None) is not None:
                 # an arrangement that says what it begins with is also told what takes its output: the

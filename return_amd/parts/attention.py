@@ -102,7 +102,11 @@ class PagedAttention:
             if self.eps is not None:
                 ops.head_rmsnorm(q, self.w_qn, float(self.eps))
                 ops.head_rmsnorm(k, self.w_kn, float(self.eps))
-            self.position.apply(q, k, step.positions)
+            # (a position encoding that asks for more of the step than positions, step_needs(), is given the step)
+            if hasattr(self.position, "step_needs"):
+                self.position.apply(q, k, step.positions, step)
+            else:
+                self.position.apply(q, k, step.positions)
             if write_cache:
                 ops.kv_write(k, v, cache.k_pool, cache.v_pool, tables.slot_mapping)
         o = rt.empty(T, Hq, D)

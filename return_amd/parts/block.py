@@ -18,7 +18,26 @@ It is registered with register_arrangement(name, cls) and named in BlockSpec.arr
 """
 from __future__ import annotations
 
+import inspect
+
 from .runtime import NormSink, ResidualSink
+
+
+_TAKES_SINK = {}
+
+
+def takes_sink(part):
+    """Whether the part's forward has a ``sink`` parameter (a part may note its last product for the
+    kernel set's measurement and still form it itself: then it is never handed a sink)."""
+    cls = type(part)
+    hit = _TAKES_SINK.get(cls)
+    if hit is None:
+        try:
+            hit = "sink" in inspect.signature(cls.forward).parameters
+        except (AttributeError, TypeError, ValueError):
+            hit = False
+        _TAKES_SINK[cls] = hit
+    return hit
 
 
 def norm_sink(h, producer, norm, consumer_first_product):
@@ -30,7 +49,7 @@ def norm_sink(h, producer, norm, consumer_first_product):
     (takes_slabs); else None: the part forms its product as it does for anyone."""
     ops = getattr(getattr(norm, "rt", None), "ops", None)
     last = getattr(producer, "last_product", None)
-    if last is None or ops is None or norm is None:
+    if last is None or ops is None or norm is None or not takes_sink(producer):
         return None
     if consumer_first_product is not None and hasattr(ops, "can_defer_norm") and \
             hasattr(norm, "weight") and hasattr(norm, "eps"):

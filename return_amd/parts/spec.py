@@ -52,12 +52,13 @@ class LayerCall:
     """One entry of the run order.
 
     block:  index into ModelSpec.blocks; the same block may be called more than once.
-    cache:  number of the cache layer this call uses (None if the mixer keeps nothing).
+    cache:  number of the cache layer this call uses (None if the mixer keeps nothing), or a
+            tuple of numbers, one for each spec of a block whose cache_spec() is a tuple.
             Two calls may name the same cache layer; only calls with writes_cache=True
             append to it, the others read what an earlier call wrote in the same step.
     """
     block: int
-    cache: Optional[int] = None
+    cache: Optional[object] = None
     writes_cache: bool = True
 
 

@@ -14,7 +14,7 @@ from tests.torch_ops import TorchOps
 
 
 def runner_for(folder, max_token, page=16, max_reside=4, **kw):
-    ec = EngineConfig(dtype="float32", page_size=page, max_token=max_token, max_reside=max_reside,
+    ec = EngineConfig(dtype="float32", check_invariants=True, page_size=page, max_token=max_token, max_reside=max_reside,
                       max_step_tokens=max(max_token, max_reside), prefill_chunk=max_token, device="cpu", **kw)
     return ModelRunner(folder, engine_config=ec, ops=TorchOps())
 
@@ -41,7 +41,7 @@ def test_generation_does_not_depend_on_the_knobs(folder_b):
     prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (1, 8, 31, 64, 100)]
     want = [plain.greedy_generate(cfg, w, p, 6) for p in prompts]
     for max_reside, chunk, max_token, page in ((4, 24, 1024, 32), (1, 1000, 256, 16), (5, 7, 416, 8)):
-        ec = EngineConfig(dtype="float32", page_size=page, max_token=max_token, max_reside=max_reside,
+        ec = EngineConfig(dtype="float32", check_invariants=True, page_size=page, max_token=max_token, max_reside=max_reside,
                           max_step_tokens=64, prefill_chunk=chunk, device="cpu")
         eng = Engine(runner=ModelRunner(folder_b, engine_config=ec, ops=TorchOps()))
         got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=6))
@@ -58,7 +58,7 @@ def test_temperature_sampling_is_reproducible_and_batch_independent(folder_a):
     prompts = [tt.random_tokens(TINY_A["vocab_size"], n, seed=n) for n in (5, 17, 33)]
     sp = [SamplingParams(temperature=0.7, max_new_tokens=10, seed=100 + i) for i in range(3)]
     def run(max_reside):
-        ec = EngineConfig(dtype="float32", page_size=16, max_token=512, max_reside=max_reside,
+        ec = EngineConfig(dtype="float32", check_invariants=True, page_size=16, max_token=512, max_reside=max_reside,
                           max_step_tokens=64, prefill_chunk=24, device="cpu", seed=7)
         return [r.output_ids for r in Engine(runner=ModelRunner(folder_a, engine_config=ec, ops=TorchOps()))
                 .generate(prompts, sp)]
@@ -141,7 +141,7 @@ def test_steps_launched_ahead_give_the_same_generation(folder_a):
               SamplingParams(temperature=0.0, max_new_tokens=7)]
 
     def run(lookahead, max_reside):
-        ec = EngineConfig(dtype="float32", page_size=16, max_token=1024, max_reside=max_reside, max_step_tokens=64,
+        ec = EngineConfig(dtype="float32", check_invariants=True, page_size=16, max_token=1024, max_reside=max_reside, max_step_tokens=64,
                           prefill_chunk=32, device="cpu", seed=3, lookahead=lookahead)
         eng = Engine(runner=ModelRunner(folder_a, engine_config=ec, ops=TorchOps()))
         out = eng.generate(prompts, params)
@@ -197,7 +197,7 @@ def test_schedule_ahead_decides_on_the_state_the_step_under_way_will_leave(folde
 
 
 def engine_for(folder, lookahead=True, **kw):
-    ec = EngineConfig(dtype="float32", page_size=16, max_token=kw.pop("max_token", 1024), max_reside=kw.pop("max_reside", 4),
+    ec = EngineConfig(dtype="float32", check_invariants=True, page_size=16, max_token=kw.pop("max_token", 1024), max_reside=kw.pop("max_reside", 4),
                       max_step_tokens=64, prefill_chunk=24, device="cpu", lookahead=lookahead, **kw)
     return Engine(runner=ModelRunner(folder, engine_config=ec, ops=TorchOps()))
 
@@ -411,3 +411,22 @@ def test_norms_are_finished_inside_the_products_in_steps_of_few_rows(folder_b):
         else:
             assert calls == {"add_norm": 0, "scaled_in": 0, "norm": 2 * L + 1}
         torch.testing.assert_close(torch.cat(got).cpu(), want, atol=2e-4, rtol=2e-4)
+
+
+def test_the_engine_checks_the_cache_after_every_step_when_asked(folder_a):
+    """EngineConfig.check_invariants: a page that is both held and free (put there by hand) is found
+    at the end of the very next step; without the option the step goes through."""
+    toks = tt.random_tokens(TINY_A["vocab_size"], 20, seed=1)
+    for on in (True, False):
+        runner = runner_for(folder_a, 256)
+        runner.engine_config.check_invariants = on
+        assert runner.engine_config.check_invariants == on
+        runner.add_request("r")
+        runner.step([StepEntry("r", toks[:10], [])])
+        held = runner.cache.live["r"].pages[0][0]
+        runner.cache.groups[0].pages._free.append(held)
+        if on:
+            with pytest.raises(AssertionError, match="both free and held|twice"):
+                runner.step([StepEntry("r", toks[10:12], [])])
+        else:
+            runner.step([StepEntry("r", toks[10:12], [])])

@@ -41,7 +41,7 @@ def test_bf16_generation_follows_plain_within_rounding(folder_b):
     from return_amd.engine import Engine
     cfg, w = plain.read_folder(folder_b)
     prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (8, 31, 64)]
-    eng = Engine(folder_b, dtype="bfloat16", page_size=16, max_token=2048, max_reside=4)
+    eng = Engine(folder_b, check_invariants=True, dtype="bfloat16", page_size=16, max_token=2048, max_reside=4)
     got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=12))
     for r, p in zip(got, prompts):
         seq = p + r.output_ids
@@ -57,7 +57,7 @@ def test_temperature_sampling_reproducible(folder_b):
     prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (1, 8, 31, 64, 100)]
     sp = [SamplingParams(temperature=0.7, max_new_tokens=20, seed=50 + i) for i in range(5)]
     def run(max_reside, chunk):
-        eng = Engine(folder_b, dtype="float32", page_size=32, max_token=4096, max_reside=max_reside,
+        eng = Engine(folder_b, check_invariants=True, dtype="float32", page_size=32, max_token=4096, max_reside=max_reside,
                      max_step_tokens=64, prefill_chunk=chunk, seed=11)
         return [r.output_ids for r in eng.generate(prompts, sp)]
     a, b = run(5, 24), run(2, 1000)
@@ -68,7 +68,7 @@ def test_top_k_top_p_through_the_engine(folder_a):
     from return_amd.engine import Engine
     cfg, w = plain.read_folder(folder_a)
     prompt = tt.random_tokens(TINY_A["vocab_size"], 12, seed=2)
-    eng = Engine(folder_a, dtype="float32", page_size=16, max_token=1024, max_reside=4)
+    eng = Engine(folder_a, check_invariants=True, dtype="float32", page_size=16, max_token=1024, max_reside=4)
     greedy = eng.generate([prompt], SamplingParams(temperature=0.0, max_new_tokens=6))[0].output_ids
     k1 = eng.generate([prompt], SamplingParams(temperature=1.5, top_k=1, max_new_tokens=6))[0].output_ids
     p0 = eng.generate([prompt], SamplingParams(temperature=1.5, top_p=0.0, max_new_tokens=6))[0].output_ids
@@ -115,7 +115,7 @@ def test_kept_sessions_on_the_gpu(folder_b, dtype):
     cfg, w = plain.read_folder(folder_b)
     V = TINY_B["vocab_size"]
     sp = SamplingParams(temperature=0.0, max_new_tokens=7)
-    eng = Engine(folder_b, dtype=dtype, page_size=16, max_token=2048, max_reside=4, max_step_tokens=64, prefill_chunk=32)
+    eng = Engine(folder_b, check_invariants=True, dtype=dtype, page_size=16, max_token=2048, max_reside=4, max_step_tokens=64, prefill_chunk=32)
     convs = {k: tt.random_tokens(V, n, seed=n) for k, n in (("a", 5), ("b", 33), ("c", 70))}
     for turn in range(3):
         ids = list(convs)
@@ -146,7 +146,7 @@ def test_kept_sessions_that_end_on_a_stop_sequence_found_a_step_late(folder_b, l
     from return_amd.engine import Engine
     cfg, w = plain.read_folder(folder_b)
     V = TINY_B["vocab_size"]
-    eng = Engine(folder_b, dtype="float32", page_size=16, max_token=2048, max_reside=4, max_step_tokens=64,
+    eng = Engine(folder_b, check_invariants=True, dtype="float32", page_size=16, max_token=2048, max_reside=4, max_step_tokens=64,
                  prefill_chunk=32, use_graphs=True, lookahead=lookahead, tune_products=False)
     convs = {k: tt.random_tokens(V, n, seed=90 + n) for k, n in (("a", 6), ("b", 31), ("c", 70), ("d", 16))}
     stop_after = {"a": 3, "b": 9, "c": 1, "d": None}           # d runs to its length

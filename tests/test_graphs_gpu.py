@@ -99,7 +99,7 @@ def test_generation_with_graphs(folder_b):
     prompts = [tt.random_tokens(TINY_B["vocab_size"], n, seed=n) for n in (1, 8, 31, 64, 100)]
     outs = []
     for use_graphs in (False, True):
-        eng = Engine(folder_b, dtype="float32", page_size=32, max_token=4096, max_reside=5,
+        eng = Engine(folder_b, check_invariants=True, dtype="float32", page_size=32, max_token=4096, max_reside=5,
                      max_step_tokens=64, prefill_chunk=24, use_graphs=use_graphs)
         outs.append([r.output_ids for r in eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=20))])
     assert outs[0] == outs[1]
@@ -121,7 +121,7 @@ def test_steps_launched_ahead_on_the_device(folder_b, dtype, use_graphs):
     def run(lookahead, stops):
         # products by rule: a request that is found finished a step late makes a batch of one row more,
         # and a measured plan may form products of 8 and of 9 rows in ways that round differently
-        eng = Engine(folder_b, dtype=dtype, page_size=16, max_token=4096, max_reside=11, max_step_tokens=128,
+        eng = Engine(folder_b, check_invariants=True, dtype=dtype, page_size=16, max_token=4096, max_reside=11, max_step_tokens=128,
                      prefill_chunk=64, use_graphs=use_graphs, lookahead=lookahead, seed=4, tune_products=False)
         params = [SamplingParams(temperature=0.0 if i % 3 else 0.9, top_k=0 if i % 2 else 30, max_new_tokens=n,
                                  seed=i, stop_ids=stops if i == 6 else [])

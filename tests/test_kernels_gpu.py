@@ -941,6 +941,28 @@ def test_sample_distribution(ops):
     assert chi2 < 30.0, (chi2, counts.tolist())
 
 
+@pytest.mark.parametrize("V", [50, 20001])
+@pytest.mark.parametrize("fill", [float("-inf"), float("nan")])
+def test_sample_of_a_row_without_a_largest_value(ops, V, fill):
+    """A row that is all -inf (or all NaN, as after an overflow upstream) has no largest value: every
+    way of choosing gives token 0 and a logprob that is no number, reads nothing beyond the row, and
+    leaves the rows beside it alone."""
+    M = 8
+    logits = rnd(M, V, seed=74, scale=2.0)
+    logits[1::2] = fill
+    temp = torch.tensor([0.0, 0.0, 1.0, 1.0, 0.8, 0.8, 1.2, 1.2], device=DEV)
+    top_k = torch.tensor([0, 0, 0, 0, 5, 5, 0, 0], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([1.0, 1.0, 1.0, 1.0, 1.0, 1.0, 0.9, 0.9], device=DEV)
+    u = torch.full((M,), 0.5, device=DEV)
+    out = ops.sample(logits, temp, top_k, top_p, u).cpu()
+    torch.cuda.synchronize()
+    lp = out[:, 1].contiguous().view(torch.float32)
+    assert out[1::2, 0].tolist() == [0, 0, 0, 0]
+    assert not torch.isfinite(lp[1::2]).any()
+    assert torch.isfinite(lp[0::2]).all() and ((out[0::2, 0] >= 0) & (out[0::2, 0] < V)).all()
+    assert int(out[0, 0]) == int(logits[0].argmax())
+
+
 def test_calls_that_do_not_fit_are_refused_before_anything_runs(ops):
     """Shapes, dtypes, devices and layouts that a kernel does not take raise KernelError on the
     host; sizes beyond a kernel's limits too."""

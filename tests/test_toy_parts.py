@@ -342,7 +342,7 @@ def generate_toy(device, ops, **options):
             toks.append(int(toy_plain_logits(cfg, weights, toks)[-1].argmax()))
         want.append(toks[len(p):])
     ec = EngineConfig(dtype="float32", page_size=4, max_token=512, max_reside=3, max_step_tokens=32,
-                      prefill_chunk=16, device=device, **options)
+                      prefill_chunk=16, device=device, check_invariants=True, **options)
     runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()}, engine_config=ec, ops=ops)
     got = Engine(runner=runner).generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=new))
     assert [r.output_ids for r in got] == want
@@ -361,4 +361,322 @@ def test_toy_generation_on_gpu(use_graphs, lookahead):
     """With graphs, the warm-up and the capture of every new (batch size, context bucket) must leave the
     requests' state alone: a step that ran twice would advance the moving averages twice."""
     runner = generate_toy("cuda:0", None, use_graphs=use_graphs, lookahead=lookahead)
+    assert bool(runner._graphs) == use_graphs
+
+
+# ------------------------------------------------------------------ a model whose mixers keep state only
+def state_only_spec(c: ToyConfig) -> ModelSpec:
+    """Two layers of the moving-average mixer and nothing else that keeps anything: no attention, so
+    the cache manager has no paged group at all, only state slots."""
+    H = c.hidden_size
+    norm = lambda name: PartSpec("rms_norm", {"size": H, "eps": c.eps}, {"weight": name})
+    mlp = lambda i: PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c.intermediate_size},
+                             {"gate_proj": f"blocks.{i}.g", "up_proj": f"blocks.{i}.u", "down_proj": f"blocks.{i}.d"})
+    ema = lambda i, decay: PartSpec("toy_ema", {"hidden_size": H, "decay": decay}, {"w": f"blocks.{i}.w"})
+    blocks = [BlockSpec.pre_norm(ema(i, d), mlp(i), norm(f"blocks.{i}.n1"), norm(f"blocks.{i}.n2"))
+              for i, d in enumerate((c.decay, 0.4))]
+    return ModelSpec(
+        architecture=c.architecture, hidden_size=H, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
+        embedding=PartSpec("token_embedding", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "embed"}),
+        positions={}, blocks=blocks, schedule=[LayerCall(0, cache=0), LayerCall(1, cache=1)],
+        final_norm=norm("final_norm"),
+        head=PartSpec("linear_head", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "head"}))
+
+
+@dataclasses.dataclass(frozen=True)
+class StateOnlyConfig(ToyConfig):
+    pass
+
+
+register_architecture("ToyStateOnlyForTests", StateOnlyConfig, state_only_spec)
+
+
+def state_only_logits(c, w, tokens):
+    T = len(tokens)
+    h = w["embed"][torch.tensor(tokens)]
+    for i, decay in enumerate((c.decay, 0.4)):
+        u = plain.rms_norm(h, w[f"blocks.{i}.n1"], c.eps) @ w[f"blocks.{i}.w"].T
+        s, ys = torch.zeros(c.hidden_size), []
+        for t in range(T):
+            s = decay * s + u[t]
+            ys.append(s)
+        h = h + torch.stack(ys)
+        x = plain.rms_norm(h, w[f"blocks.{i}.n2"], c.eps)
+        g = x @ w[f"blocks.{i}.g"].T
+        h = h + (g * torch.sigmoid(g) * (x @ w[f"blocks.{i}.u"].T)) @ w[f"blocks.{i}.d"].T
+    return plain.rms_norm(h, w["final_norm"], c.eps) @ w["head"].T
+
+
+def run_state_only(device, ops, **options):
+    """Replay under every cut, then greedy generation through the entry point: a model without a single
+    page of cache goes through admission, the step's tables, the step function and the scheduler."""
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    cfg = StateOnlyConfig.from_dict(dict(TOY, architectures=["ToyStateOnlyForTests"]))
+    weights = random_weights(state_only_spec(cfg), seed=6, std=0.08, norm_jitter=0.05, dtype="float32")
+    reqs = {rid: tt.random_tokens(cfg.vocab_size, n, seed=ord(rid)) for rid, n in
+            {"a": 40, "b": 7, "c": 23, "d": 61, "e": 1}.items()}
+    want = {rid: state_only_logits(cfg, weights, toks) for rid, toks in reqs.items()}
+    for cut in (tt.whole, tt.portions, tt.mixed):
+        steps = cut(reqs)
+        ec = EngineConfig(dtype="float32", page_size=4, max_token=64, max_reside=4, max_step_tokens=256,
+                          prefill_chunk=256, device=device, check_invariants=True)
+        runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()}, engine_config=ec, ops=ops)
+        assert len(runner.cache.groups) == 0 and len(runner.cache.state_layers) == 2
+        got = tt.run_in_process(runner, steps)
+        for rid, toks in reqs.items():
+            for p in range(len(toks)):
+                torch.testing.assert_close(got[(rid, p)], want[rid][p], atol=3e-4, rtol=3e-4,
+                                           msg=lambda m: f"{cut.__name__} request {rid} position {p}: {m}")
+        assert runner.cache.free_slots() == 4
+    prompts = [tt.random_tokens(cfg.vocab_size, n, seed=90 + n) for n in (9, 1, 30, 17, 4)]
+    new = 20
+    expect = []
+    for p in prompts:
+        toks = list(p)
+        for _ in range(new):
+            toks.append(int(state_only_logits(cfg, weights, toks)[-1].argmax()))
+        expect.append(toks[len(p):])
+    # max_token is as small as it may be: nothing here is held in pages, so requests of any length are let in
+    ec = EngineConfig(dtype="float32", page_size=4, max_token=4, max_reside=3, max_step_tokens=32, prefill_chunk=16,
+                      device=device, check_invariants=True, **options)
+    runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()}, engine_config=ec, ops=ops)
+    out = Engine(runner=runner).generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=new))
+    assert [r.output_ids for r in out] == expect
+    assert not runner.cache.live and runner.cache.free_slots() == 3
+    return runner
+
+
+def test_state_only_model_on_cpu_stand_in():
+    from tests.torch_ops import TorchOps
+    run_state_only("cpu", TorchOps(), lookahead=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_state_only_model_on_gpu(use_graphs):
+    runner = run_state_only("cuda:0", None, use_graphs=use_graphs)
+    assert bool(runner._graphs) == use_graphs
+
+
+# ------------------------------------------------------------------ a mixer that keeps two things, a weight with a law
+# of its own, and a position encoding with a second axis
+class ConvThenAttention:
+    """A short causal convolution over the tokens (taps that are positive and sum to one), then attention over
+    the paged cache: the layer keeps paged keys and values AND a state of fixed size, the last K - 1 inputs."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        from return_amd.parts.attention import PagedAttention
+        return dict(PagedAttention.tensor_shapes(params), taps=(params["taps"],))
+
+    @staticmethod
+    def random_init(params, role):
+        from return_amd.parts.attention import PagedAttention
+        if role == "taps":
+            # a law of its own: no normal draw gives positive numbers that sum to one
+            draw = lambda shape, gen: torch.randn(*shape, generator=gen).softmax(-1)
+            draw.keep_dtype = True                         # and they stay 32-bit in a bfloat16 model folder
+            return draw
+        return PagedAttention.random_init(params, role)
+
+    def __init__(self, params, tensors, rt, shared=None):
+        from return_amd.parts.attention import PagedAttention
+        self.rt, self.h, self.k = rt, int(params["hidden_size"]), int(params["taps"])
+        self.attention = PagedAttention(params, {r: t for r, t in tensors.items() if r != "taps"}, rt, shared)
+        assert tensors["taps"].dtype == torch.float32
+        self.taps = tensors["taps"].to(rt.device).float()             # taps[j] weighs the input j tokens back
+
+    def cache_spec(self):
+        return (self.attention.cache_spec(), StateSpec((("tail", (self.k - 1, self.h), "float32"),)))
+
+    def step_needs(self):
+        return self.attention.step_needs()
+
+    def forward(self, x, step, cache, write_cache=True):
+        paged, state = cache
+        tail_of = state.tensors["tail"]
+        back = self.taps.flip(0)[None, :, None]                       # oldest input first
+        if step.all_decode:
+            window = torch.cat([tail_of.index_select(0, step.slot_ids), x.float()[:, None, :]], dim=1)
+            y = (window * back).sum(1)
+            if write_cache:
+                tail_of.index_copy_(0, step.slot_ids.long(), window[:, 1:].contiguous())
+        else:
+            y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            for i in range(step.n_seqs):
+                a, b = step.cu_q_host[i], step.cu_q_host[i + 1]
+                slot = step.slot_ids_host[i]
+                seq = torch.cat([tail_of[slot], x[a:b].float()], dim=0)
+                y[a:b] = (seq.unfold(0, self.k, 1) * self.taps.flip(0)[None, None, :]).sum(-1)
+                if write_cache:
+                    tail_of[slot] = seq[-(self.k - 1):]
+        return self.attention.forward(y.to(x.dtype).contiguous(), step, paged, write_cache)
+
+
+class GridFade:
+    """A position encoding of two axes: keys fade with the token's position AND with its row on a grid, an
+    integer that the request brings with every token (the step's token column "row")."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        return {}
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.along, self.down = float(params["along"]), float(params["down"])
+
+    def step_needs(self):
+        return {"token_columns": ("row",)}
+
+    def apply(self, q, k, positions, step):
+        if k is not None:
+            row = step.token_columns["row"]
+            fade = 1.0 / ((1.0 + positions.float() / self.along) * (1.0 + row.float() / self.down))
+            k.mul_(fade.to(k.dtype)[:, None, None])
+
+
+register_part("mixer", "toy_conv_then_attention", ConvThenAttention)
+register_part("position", "toy_grid_fade", GridFade)
+
+
+@dataclasses.dataclass(frozen=True)
+class HybridConfig(ToyConfig):
+    taps: int = 3
+
+
+def hybrid_spec(c: HybridConfig) -> ModelSpec:
+    H = c.hidden_size
+    norm = lambda name: PartSpec("rms_norm", {"size": H, "eps": c.eps}, {"weight": name})
+    mlp = lambda i: PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c.intermediate_size},
+                             {"gate_proj": f"blocks.{i}.g", "up_proj": f"blocks.{i}.u", "down_proj": f"blocks.{i}.d"})
+
+    def attn(i, kind, position, **more):
+        names = {r: f"blocks.{i}.{r}" for r in ("q_proj", "k_proj", "v_proj", "o_proj") + tuple(more.pop("roles", ()))}
+        return PartSpec(kind, dict({"hidden_size": H, "num_heads": c.heads, "num_kv_heads": c.kv_heads,
+                                    "head_dim": c.head_dim, "scale": None, "window": None, "qk_norm_eps": None,
+                                    "position": position}, **more), names)
+    blocks = [BlockSpec.pre_norm(attn(0, "toy_conv_then_attention", "grid", taps=c.taps, roles=("taps",)), mlp(0),
+                                 norm("blocks.0.n1"), norm("blocks.0.n2")),
+              BlockSpec.pre_norm(attn(1, "attention", "grid"), mlp(1), norm("blocks.1.n1"), norm("blocks.1.n2"))]
+    return ModelSpec(
+        architecture=c.architecture, hidden_size=H, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
+        embedding=PartSpec("token_embedding", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "embed"}),
+        positions={"grid": PartSpec("toy_grid_fade", {"along": 40.0, "down": 3.0})}, blocks=blocks,
+        # the first call names two cache layers, one for each thing its mixer keeps
+        schedule=[LayerCall(0, cache=(0, 1)), LayerCall(1, cache=2)], final_norm=norm("final_norm"),
+        head=PartSpec("linear_head", {"vocab_size": c.vocab_size, "hidden_size": H}, {"weight": "head"}))
+
+
+register_architecture("ToyHybridForTests", HybridConfig, hybrid_spec)
+
+
+def grid_rows(n, width=4, start=0):
+    """The rows of n tokens laid out on a grid of the given width, then counting on."""
+    return [start + i // width for i in range(n)]
+
+
+def hybrid_logits(c, w, tokens, rows):
+    T, D = len(tokens), c.head_dim
+    pos, row = torch.arange(T), torch.tensor(rows)
+    h = w["embed"][torch.tensor(tokens)]
+    fade = 1.0 / ((1.0 + pos.float() / 40.0) * (1.0 + row.float() / 3.0))
+
+    def attention(x, i):
+        p = f"blocks.{i}."
+        q = (x @ w[p + "q_proj"].T).view(T, -1, D)
+        k = (x @ w[p + "k_proj"].T).view(T, -1, D) * fade[:, None, None]
+        v = (x @ w[p + "v_proj"].T).view(T, -1, D)
+        return plain.causal_attention(q, k, v, pos, pos, D ** -0.5, None).reshape(T, -1) @ w[p + "o_proj"].T
+
+    def swiglu(x, i):
+        g = x @ w[f"blocks.{i}.g"].T
+        return (g * torch.sigmoid(g) * (x @ w[f"blocks.{i}.u"].T)) @ w[f"blocks.{i}.d"].T
+
+    x = plain.rms_norm(h, w["blocks.0.n1"], c.eps)
+    taps = w["blocks.0.taps"]
+    padded = torch.cat([torch.zeros(c.taps - 1, c.hidden_size), x])
+    y = sum(taps[j] * padded[c.taps - 1 - j: c.taps - 1 - j + T] for j in range(c.taps))
+    h = h + attention(y, 0)
+    h = h + swiglu(plain.rms_norm(h, w["blocks.0.n2"], c.eps), 0)
+    h = h + attention(plain.rms_norm(h, w["blocks.1.n1"], c.eps), 1)
+    h = h + swiglu(plain.rms_norm(h, w["blocks.1.n2"], c.eps), 1)
+    return plain.rms_norm(h, w["final_norm"], c.eps) @ w["head"].T
+
+
+def run_hybrid(device, ops, **options):
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    cfg = HybridConfig.from_dict(dict(TOY, architectures=["ToyHybridForTests"], taps=3))
+    weights = random_weights(hybrid_spec(cfg), seed=8, std=0.08, norm_jitter=0.05, dtype="float32")
+    taps = weights["blocks.0.taps"]
+    assert taps.dtype == torch.float32 and bool((taps > 0).all()) and abs(float(taps.sum()) - 1.0) < 1e-6
+    # in a bfloat16 model the taps stay as their law drew them
+    assert random_weights(hybrid_spec(cfg), seed=8, dtype="bfloat16")["blocks.0.taps"].dtype == torch.float32
+    reqs = {rid: tt.random_tokens(cfg.vocab_size, n, seed=ord(rid)) for rid, n in
+            {"a": 40, "b": 7, "c": 23, "d": 61, "e": 1}.items()}
+    rows = {rid: grid_rows(len(toks), start=ord(rid) % 3) for rid, toks in reqs.items()}
+    want = {rid: hybrid_logits(cfg, weights, toks, rows[rid]) for rid, toks in reqs.items()}
+    for cut in (tt.whole, tt.portions, tt.mixed):
+        steps = cut(reqs)
+        at = {rid: 0 for rid in reqs}
+        for s in steps:                                   # every entry brings its tokens' rows
+            for e in s["entries"]:
+                n = len(e["tokens"])
+                e["columns"] = {"row": rows[e["id"]][at[e["id"]]:at[e["id"]] + n]}
+                at[e["id"]] += n
+        ec = EngineConfig(dtype="float32", page_size=4, max_token=tt.peak_tokens(steps), max_reside=4,
+                          max_step_tokens=256, prefill_chunk=256, device=device, check_invariants=True)
+        runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()}, engine_config=ec, ops=ops)
+        assert runner.builder.token_columns == ("row",)
+        assert len(runner.cache.groups) == 1 and sorted(runner.cache.state_layers) == [1]
+        assert runner.cache.groups[0].layers == [0, 2]
+        got = tt.run_in_process(runner, steps)
+        for rid, toks in reqs.items():
+            for p in range(len(toks)):
+                torch.testing.assert_close(got[(rid, p)], want[rid][p], atol=3e-4, rtol=3e-4,
+                                           msg=lambda m: f"{cut.__name__} request {rid} position {p}: {m}")
+    # generation: the prompt's rows come with the request, the generated tokens' rows count on from the last
+    prompts = [tt.random_tokens(cfg.vocab_size, n, seed=40 + n) for n in (9, 1, 30, 17, 4)]
+    new = 16
+    columns, expect = [], []
+    for p in prompts:
+        r = grid_rows(len(p))
+        columns.append({"row": r})
+        toks, r = list(p), list(r)
+        for _ in range(new):
+            toks.append(int(hybrid_logits(cfg, weights, toks, r)[-1].argmax()))
+            r.append(r[-1] + 1)
+        expect.append(toks[len(p):])
+    ec = EngineConfig(dtype="float32", page_size=4, max_token=512, max_reside=3, max_step_tokens=32, prefill_chunk=16,
+                      device=device, check_invariants=True, **options)
+    runner = ModelRunner(config=cfg, weights={k: v.clone() for k, v in weights.items()}, engine_config=ec, ops=ops)
+    eng = Engine(runner=runner)
+    out = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=new), token_columns=columns)
+    assert [r.output_ids for r in out] == expect
+    # without its rows a request is computed as if every token's row were its position: other logits
+    from return_amd.engine import StepEntry
+    p = prompts[2]
+    rows_of = {"with": {"row": grid_rows(len(p))}, "without": None, "as_positions": {"row": list(range(len(p)))}}
+    for rid in rows_of:
+        runner.add_request(rid)
+    got = {rid: runner.step([StepEntry(rid, p, [len(p) - 1], cols)])[0].cpu() for rid, cols in rows_of.items()}
+    for rid in rows_of:
+        runner.free_request(rid)
+    torch.testing.assert_close(got["with"], hybrid_logits(cfg, weights, p, grid_rows(len(p)))[-1], atol=3e-4, rtol=3e-4)
+    assert torch.equal(got["without"], got["as_positions"])
+    assert float((got["with"] - got["without"]).abs().max()) > 1e-2
+    with pytest.raises(ValueError, match="column"):
+        eng.submit(prompts[0], token_columns={"depth": [0] * len(prompts[0])})
+    return runner
+
+
+def test_layer_with_pages_and_state_and_a_second_position_axis_on_cpu_stand_in():
+    from tests.torch_ops import TorchOps
+    run_hybrid("cpu", TorchOps(), lookahead=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_layer_with_pages_and_state_and_a_second_position_axis_on_gpu(use_graphs):
+    runner = run_hybrid("cuda:0", None, use_graphs=use_graphs)
     assert bool(runner._graphs) == use_graphs

@@ -64,18 +64,36 @@ def _run(lib, c, static, warm=False):
     return rc, out
 
 
+def _plain(c, lengths):
+    """Softmax attention of every request's one query over its keys, gathered from the pages, in 32-bit."""
+    out = torch.zeros(c["n"], c["Hq"], c["D"])
+    kp, vp, table = c["kp"].float().cpu(), c["vp"].float().cpu(), c["page_table"].cpu().tolist()
+    q, cu, P, G = c["q"].float().cpu(), c["cu_pages"].cpu().tolist(), c["P"], c["Hq"] // c["Hkv"]
+    for i, n in enumerate(lengths):
+        pages = table[cu[i]:cu[i + 1]]
+        k = torch.cat([kp[p] for p in pages], dim=1)[:, :n]            # [Hkv, n, D]
+        v = torch.cat([vp[p] for p in pages], dim=1)[:, :n]
+        for h in range(c["Hq"]):
+            w = ((k[h // G] @ q[i, h]) * c["D"] ** -0.5).softmax(0)
+            out[i, h] = w @ v[h // G]
+    return out
+
+
 def test_decode_attention_without_allocation_two_calls_in_a_row():
     torch.cuda.set_device(0)
     lib = _lib()
-    big = _case([900, 130, 64, 517, 1, 333], Hq=8, Hkv=2, D=128, P=16, split=128, seed=1)
-    small = _case([70, 200], Hq=6, Hkv=3, D=64, P=16, split=64, seed=2)
-    for c in (big, small):                      # the second call finds the first one's partial sums in the buffer
+    lengths = {"big": [900, 130, 64, 517, 1, 333], "small": [70, 200]}
+    big = _case(lengths["big"], Hq=8, Hkv=2, D=128, P=16, split=128, seed=1)
+    small = _case(lengths["small"], Hq=6, Hkv=3, D=64, P=16, split=64, seed=2)
+    for name, c in (("big", big), ("small", small)):   # the second call finds the first one's partial sums in the buffer
         rc, want = _run(lib, c, static=False)
         assert rc == 0
         rc, got = _run(lib, c, static=True, warm=c is small)
         assert rc == 0
         assert torch.equal(got, want)
         assert want.float().abs().max() > 0
+        # and both against a 32-bit evaluation that shares nothing with the library
+        torch.testing.assert_close(got.float().cpu(), _plain(c, lengths[name]), atol=2e-2, rtol=2e-2)
 
 
 def test_decode_attention_without_allocation_refuses_what_does_not_fit():

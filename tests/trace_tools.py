@@ -113,7 +113,7 @@ def run_in_process(runner, steps):
             if not runner.is_live(e["id"]):
                 runner.add_request(e["id"])
                 pos[e["id"]] = 0
-            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"], e.get("columns")))
         logits = runner.step(entries)
         if logits is not None:
             logits = logits.float().cpu()
