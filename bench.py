@@ -211,6 +211,49 @@ def release(runner, ids):
         runner.free_request(rid)
 
 
+def hbm_roofline(cfg, elt, batch, mean_ctx, ms, peaks=None):
+    """Bytes a decode step has to read (every weight once, the cache of `batch` live requests of mean_ctx
+    tokens) over its time, against the published read rate and the one measured in this run."""
+    step_bytes = weight_bytes(cfg, elt) + batch * mean_ctx * kv_bytes_per_token(cfg, elt)
+    got = step_bytes / (ms * 1e-3) / 1e9
+    r = {"bound": "hbm", "achieved": round(got, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+         "frac": round(got / PEAK_HBM_GBS, 4)}
+    if peaks:
+        r["measured_peak"] = peaks["read_GBs"]
+        r["frac_of_measured"] = round(got / peaks["read_GBs"], 4)
+    return r
+
+
+def prefill_record(cfg, dtype, tokens, secs, count=1, peaks=None, flops=None):
+    """tok/s of `count` prompts of `tokens` tokens in `secs`, with the fraction of the published matrix rate
+    and of the library product's rate measured in this run."""
+    f = count * prefill_flops(cfg, tokens) if flops is None else flops
+    r = {"value": round(count * tokens / secs, 1), "tokens": count * tokens, "ms": round(secs * 1e3, 3),
+         "frac": round(f / secs / PEAK_FLOPS[dtype], 4)}
+    if peaks:
+        r["measured_peak_TFLOPs"] = peaks["product_TFLOPs"]
+        r["frac_of_measured"] = round(f / secs / (peaks["product_TFLOPs"] * 1e12), 4)
+    return r
+
+
+def decode_point(runner, cfg, elt, batch, ctx, steps, warmup, peaks=None, kernels=False):
+    """Seats `batch` requests at ctx tokens, times `steps` decode steps after `warmup`, gives the requests
+    back. tok/s, ms a step and the roofline; with kernels the step's time by kernel from a pass of its own."""
+    ids = seat_requests(runner, batch, ctx)
+    secs = decode_steps(runner, ids, steps, warmup, cfg.vocab_size)
+    ms = secs / steps * 1e3
+    out = {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4)}
+    out.update(hbm_roofline(cfg, elt, batch, ctx + warmup + (steps + 1) / 2.0, ms, peaks))
+    if kernels:
+        def one_step():
+            t = runner.decode_launch(ids, None, [0.0] * batch, [0] * batch, [1.0] * batch, [0.0] * batch,
+                                     feed_rows=list(range(batch)))
+            runner.decode_collect(t)
+        out["kernels"] = kernel_split(one_step, 4)
+    release(runner, ids)
+    return out
+
+
 # the two other shapes of the benchmark, each with its own workload
 QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64,
@@ -237,20 +280,45 @@ def continuous_4b(args):
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_4B, use_graphs=not args.no_graphs,
                                tune_products=not args.no_tune, defer_norms=not args.no_defer_norms,
                                max_token=n * 4608, max_step_tokens=512 + n, prefill_chunk=512)
+    elt = 2 if args.dtype == "bfloat16" else 4
+    peaks = measured_peaks(runner, args.dtype)
     eng = Engine(runner=runner)
     rnd = random.Random(0)
     prompts = [[rnd.randrange(cfg.vocab_size) for _ in range(rnd.randint(64, 4096))] for _ in range(n)]
     params = [SamplingParams(temperature=0.0, max_new_tokens=rnd.randint(32, 512)) for _ in range(n)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    out = eng.generate(prompts, params)
+    reqs = [eng.submit(p, sp) for p, sp in zip(prompts, params)]
+    # the steps one by one, as Engine.generate runs them; beside each what it had to read, so that the run's
+    # last stretch, in which every prompt is done and the steps only decode, gets a roofline of its own
+    log = []                                    # (seconds since t0, brought a prompt portion, requests, cached tokens)
+    while eng.scheduler.has_work() or eng._in_flight is not None:
+        before = eng.prefill_tokens
+        live = [runner.cache.seq_len(rid) for rid in runner.cache.live]
+        eng.step()
+        log.append((time.perf_counter() - t0, eng.prefill_tokens != before, len(live), sum(live)))
     torch.cuda.synchronize()
     secs = time.perf_counter() - t0
+    out = [eng.result_of(r) for r in reqs]
     if any(r.num_tokens != p.max_new_tokens for r, p in zip(out, params)):
         raise RuntimeError("a request ended early")
     runner.cache.check_invariants()
     made, read = sum(r.num_tokens for r in out), sum(map(len, prompts))
     flops = 2.0 * (read + made) * (weight_bytes(cfg, 1) - cfg.vocab_size * cfg.hidden_size)
+    first = len(log)
+    while first > 0 and not log[first - 1][1]:
+        first -= 1
+    tail = log[first:-1] if len(log) - first > 2 else []       # (the very last call only collects)
+    tail_record = None
+    if tail:
+        t_tail = tail[-1][0] - (log[first - 1][0] if first else 0.0)
+        ms = t_tail / len(tail) * 1e3
+        mean_batch = sum(x[2] for x in tail) / len(tail)
+        mean_ctx = sum(x[3] for x in tail) / max(1.0, sum(x[2] for x in tail))
+        tail_record = dict(hbm_roofline(cfg, elt, mean_batch, mean_ctx, ms, peaks), steps=len(tail),
+                           ms_per_step=round(ms, 4), mean_batch=round(mean_batch, 1), mean_context=round(mean_ctx, 1))
+    # a decode step of 64 requests at 2,048 tokens on this shape, with its time by kernel (outside the timed run)
+    decode64 = decode_point(runner, cfg, elt, 64, 2048, 16, 4, peaks, kernels=True)
     return {"metric": "generated tok/s, continuous batching (Qwen3-4B shape, random weights)",
             "value": round(made / secs, 1), "unit": "tok/s", "n_gpus": 1, "steps": eng.steps, "warmup": 0,
             "ms_per_step": round(secs / eng.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
@@ -258,8 +326,11 @@ def continuous_4b(args):
             "config": shape_of(cfg, model="Qwen3-4B shape", global_batch=n, prompt_tokens=read, new_tokens=made,
                                prefill_chunk=512, max_context=4608, hip_graphs=not args.no_graphs,
                                weights="random N(0,0.02)"),
-            "seconds": round(secs, 3), "prompt_tok_s": round(read / secs, 1),
-            "linear_flops_frac": round(flops / secs / PEAK_FLOPS[args.dtype], 4)}
+            "seconds": round(secs, 3), "measured": peaks,
+            # the whole run as matrix work: prompt and generated tokens through every projection
+            "prefill": dict(prefill_record(cfg, args.dtype, read, secs, peaks=peaks, flops=flops), new_tokens=made),
+            "roofline": tail_record,            # of the steps after the last prompt portion, which only decode
+            "decode_b64_ctx2048": decode64}
 
 
 def long_32b(args):
@@ -275,6 +346,7 @@ def long_32b(args):
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_32B, std=0.01, use_graphs=not args.no_graphs,
                                tune_products=not args.no_tune, defer_norms=not args.no_defer_norms,
                                max_token=n * (ctx + 512) + long_ctx, max_step_tokens=ctx, prefill_chunk=ctx)
+    peaks = measured_peaks(runner, args.dtype)
     eng = Engine(runner=runner)
     rnd = random.Random(1)
     prompts = [[rnd.randrange(cfg.vocab_size) for _ in range(ctx)] for _ in range(n)]
@@ -294,8 +366,6 @@ def long_32b(args):
     runner.cache.check_invariants()
     steps, made = eng.steps - n0, eng.decode_tokens - d0
     ms_step = (t2 - t1) / steps * 1e3
-    step_bytes = weight_bytes(cfg, elt) + n * (ctx + new / 2.0) * kv_bytes_per_token(cfg, elt)
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
     long_prompt = [rnd.randrange(cfg.vocab_size) for _ in range(long_ctx)]
     best = None
     for _ in range(2):
@@ -306,10 +376,8 @@ def long_32b(args):
         dt = time.perf_counter() - t3
         best = dt if best is None else min(best, dt)
 
-    def pre(tokens, secs, count):
-        f = count * prefill_flops(cfg, tokens)
-        return {"value": round(count * tokens / secs, 1), "tokens": count * tokens, "ms": round(secs * 1e3, 1),
-                "frac": round(f / secs / PEAK_FLOPS[args.dtype], 4)}
+    # the same decode step again with its time by kernel (a pass of its own, outside the timed run)
+    again = decode_point(runner, cfg, elt, n, ctx, 8, 2, peaks, kernels=True)
     return {"metric": "decode tok/s at batch 16, 8,192-token prompts (Qwen3-32B shape, random weights)",
             "value": round(made / (t2 - t1), 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
             "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -317,37 +385,34 @@ def long_32b(args):
             "config": shape_of(cfg, model="Qwen3-32B shape", global_batch=n, seq_len=ctx, new_tokens=new,
                                long_prompt=long_ctx, prefill_chunk=ctx, hip_graphs=not args.no_graphs,
                                weights="random N(0,0.01)"),
-            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(achieved / PEAK_HBM_GBS, 4)},
-            "prefill": pre(ctx, t1 - t0, n), "prefill_long": pre(long_ctx, best, 1)}
+            "measured": peaks, "roofline": hbm_roofline(cfg, elt, n, ctx + new / 2.0, ms_step, peaks),
+            "prefill": prefill_record(cfg, args.dtype, ctx, t1 - t0, n, peaks),
+            "prefill_long": prefill_record(cfg, args.dtype, long_ctx, best, 1, peaks),
+            "kernels": again.pop("kernels")}
 
 
 def contexts_8b(args):
-    """The 8B shape at further context lengths: decode at batch 1, 8 and 64 over contexts of 8,192 and
-    32,768 tokens (batch 64 at 32,768 would need 309 GB of cache and is left out), each with the
-    fraction of the read roofline, a prefill of 16,384 tokens in one portion, and what sampling with
-    top_p = 0.9 costs at 64 rows of this vocabulary beside greedy sampling. value: decode tok/s at
-    batch 8 over 8,192 tokens."""
+    """The 8B shape at further context lengths: decode at batch 1, 8, 16, 32 and 64 over contexts of 8,192
+    and 32,768 tokens (batch 64 at 32,768 would need 309 GB of cache and is left out), each with the
+    fraction of the read roofline, published and measured in this run; prompts of 16,384 and 32,768
+    tokens in one portion and of 32,768 in portions of 8,192; and what sampling with top_p = 0.9 costs at
+    64 rows of this vocabulary beside greedy sampling. value: decode tok/s at batch 8 over 8,192 tokens."""
     import torch
     from return_amd.engine import StepEntry
     elt = 2 if args.dtype == "bfloat16" else 4
     points = {}
-    cfg = runner = None
-    for ctx, batches in ((8192, (1, 8, 64)), (32768, (1, 8))):
+    cfg = runner = peaks = kernels = None
+    k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+    for ctx, batches in ((8192, (1, 8, 16, 32, 64)), (32768, (1, 8, 16, 32))):
         del runner
         torch.cuda.empty_cache()
         cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(batches), use_graphs=not args.no_graphs,
                                    tune_products=not args.no_tune, max_token=max(batches) * (ctx + 256))
+        peaks = peaks or measured_peaks(runner, args.dtype)
         for b in batches:
-            ids = seat_requests(runner, b, ctx)
-            k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
-            secs = decode_steps(runner, ids, k, w, cfg.vocab_size)
-            release(runner, ids)
-            ms = secs / k * 1e3
-            step_bytes = weight_bytes(cfg, elt) + b * (ctx + w + (k + 1) / 2.0) * kv_bytes_per_token(cfg, elt)
-            got = step_bytes / (ms * 1e-3) / 1e9
-            points[f"decode_b{b}_ctx{ctx}"] = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4),
-                                              "GBs": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4)}
+            pt = decode_point(runner, cfg, elt, b, ctx, k, w, peaks, kernels=(ctx == 8192 and b == 8))
+            kernels = pt.pop("kernels", kernels)
+            points[f"decode_b{b}_ctx{ctx}"] = pt
     # ---- sampling at 64 rows of the full vocabulary: greedy, temperature 1 alone, with top_p 0.9, with top_k 50;
     # on flat rows (N(0, 3): thresholds are searched over the whole row) and on rows shaped like a language
     # model's (a bulk of N(0, 1.5), 500 tokens at 10 to 20 and one at 24: thresholds from the list of the largest)
@@ -371,33 +436,63 @@ def contexts_8b(args):
                 best = dt if best is None else min(best, dt)
             sampling[prefix + name + "_us"] = round(best * 1e6, 1)
     del flat, peaked
-    # ---- one prompt of 16,384 tokens in one portion
-    n = 16384
+    # ---- long prompts: 16,384 and 32,768 tokens in one portion each, 32,768 in portions of 8,192
     del runner
     torch.cuda.empty_cache()
-    cfg, runner = build_runner(args.layers, args.dtype, max_reside=2, use_graphs=False, tune_products=False,
-                               max_token=n + 256, max_step_tokens=n, prefill_chunk=n)
-    prompt = [(13 * i + 5) % cfg.vocab_size for i in range(n)]
-    times = []
-    for _ in range(3):
-        runner.add_request("p")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        runner.step([StepEntry("p", prompt, [n - 1])]).sum().item()
-        times.append(time.perf_counter() - t0)
-        runner.free_request("p")
-    pf = min(times[1:])
+    longest = 32768
+    cfg, runner = build_runner(args.layers, args.dtype, max_reside=2, use_graphs=False, tune_products=not args.no_tune,
+                               max_token=longest + 256, max_step_tokens=longest, prefill_chunk=longest)
+    prefills = {}
+    for n, portion in ((16384, 16384), (longest, longest), (longest, 8192)):
+        prompt = [(13 * i + 5) % cfg.vocab_size for i in range(n)]
+        times = []
+        for _ in range(3):
+            runner.add_request("p")
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for at in range(0, n, portion):
+                last = at + portion >= n
+                out = runner.step([StepEntry("p", prompt[at:at + portion], [portion - 1] if last else [])])
+            out.sum().item()
+            times.append(time.perf_counter() - t0)
+            runner.free_request("p")
+        name = f"prefill_{n}" + ("" if portion == n else f"_in_portions_of_{portion}")
+        prefills[name] = prefill_record(cfg, args.dtype, n, min(times[1:]), 1, peaks)
     head = points["decode_b8_ctx8192"]
-    return {"metric": "decode tok/s at batch 8 over 8,192-token contexts (Qwen3-8B shape, random weights)",
-            "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": max(8, min(args.steps, 32)),
-            "warmup": min(args.warmup, 4), "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+    line = {"metric": "decode tok/s at batch 8 over 8,192-token contexts (Qwen3-8B shape, random weights)",
+            "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": k, "warmup": w,
+            "ms_per_step": head["ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic",
             "config": shape_of(cfg, model="Qwen3-8B shape", global_batch=8, seq_len=8192, hip_graphs=not args.no_graphs,
                                weights="random N(0,0.02)"),
-            "points": points, "sampling_64_rows": sampling,
-            "prefill_16384": {"value": round(n / pf, 1), "tokens": n, "ms": round(pf * 1e3, 2),
-                              "frac": round(prefill_flops(cfg, n) / pf / PEAK_FLOPS[args.dtype], 4)}}
+            "measured": peaks, "roofline": {x: head[x] for x in head if x not in ("tok_s", "ms_per_step")},
+            "kernels": kernels, "points": points, "sampling_64_rows": sampling}
+    line.update(prefills)
+    return line
+
+
+def decode_shape(args, raw, name, std):
+    """Decode at batch 1, 8 and 64 over 2,048-token prefixes on another shape of the family, as the headline
+    run does on the 8B shape: tok/s, ms a step and the read roofline (published and measured in this run) per
+    point, the time by kernel at batch 8. value: decode tok/s at batch 8."""
+    elt = 2 if args.dtype == "bfloat16" else 4
+    cfg, runner = build_runner(0, args.dtype, 64, raw=raw, std=std, use_graphs=not args.no_graphs,
+                               tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
+    peaks = measured_peaks(runner, args.dtype)
+    k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+    points = {f"decode_b{b}": decode_point(runner, cfg, elt, b, CONTEXT, k, w, peaks, kernels=(b == 8))
+              for b in (1, 8, 64)}
+    head = points["decode_b8"]
+    kernels = head.pop("kernels")
+    return {"metric": f"decode tok/s ({name} shape, random weights)", "value": head["tok_s"], "unit": "tok/s",
+            "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic",
+            "config": shape_of(cfg, model=f"{name} shape", global_batch=8, seq_len=CONTEXT, max_context=MAX_CONTEXT,
+                               hip_graphs=not args.no_graphs, weights=f"random N(0,{std})"),
+            "measured": peaks, "roofline": {x: head[x] for x in head if x not in ("tok_s", "ms_per_step")},
+            "kernels": kernels, "points": points}
 
 
 def products_8b(args):
@@ -427,7 +522,8 @@ def products_8b(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="decode_8b",
-                    choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b"],
+                    choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b", "decode_4b",
+                             "decode_32b"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -455,7 +551,9 @@ def main():
         return 1
     if args.workload != "decode_8b":
         print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
-                          "contexts_8b": contexts_8b, "products_8b": products_8b}[args.workload](args)))
+                          "contexts_8b": contexts_8b, "products_8b": products_8b,
+                          "decode_4b": lambda a: decode_shape(a, QWEN3_4B, "Qwen3-4B", 0.02),
+                          "decode_32b": lambda a: decode_shape(a, QWEN3_32B, "Qwen3-32B", 0.01)}[args.workload](args)))
         return 0
     elt = 2 if args.dtype == "bfloat16" else 4
     cfg, runner = build_runner(args.layers, args.dtype, max_reside=max(64, args.batch),
@@ -464,17 +562,8 @@ def main():
     V = cfg.vocab_size
 
     def roofline(batch, ms, new_before, steps):
-        """Bytes a decode step has to read (every weight once, the cache of the live requests at their
-        mean length over the timed steps) over its time, against the published and the measured read rate."""
-        mean_ctx = CONTEXT + new_before + (steps + 1) / 2.0
-        step_bytes = weight_bytes(cfg, elt) + batch * mean_ctx * kv_bytes_per_token(cfg, elt)
-        got = step_bytes / (ms * 1e-3) / 1e9
-        r = {"bound": "hbm", "achieved": round(got, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-             "frac": round(got / PEAK_HBM_GBS, 4)}
-        if peaks:
-            r["measured_peak"] = peaks["read_GBs"]
-            r["frac_of_measured"] = round(got / peaks["read_GBs"], 4)
-        return r
+        """The step's roofline at the mean length of the live requests over the timed steps."""
+        return hbm_roofline(cfg, elt, batch, CONTEXT + new_before + (steps + 1) / 2.0, ms, peaks)
 
     peaks = None if args.no_points else measured_peaks(runner, args.dtype)
 
@@ -495,14 +584,13 @@ def main():
 
     points, point_rooflines, prefill, prefill_kernels = {}, {}, None, None
     if not args.no_points:
-        for b in (1, 64):
-            ids = seat_requests(runner, b, CONTEXT)
+        for b in (1, 16, 32, 64):
+            if b == args.batch:
+                continue
             k = max(8, min(args.steps, 32))
-            w = min(args.warmup, 4)
-            s = decode_steps(runner, ids, k, w, V)
-            release(runner, ids)
-            points[f"decode_b{b}"] = round(b * k / s, 1)
-            point_rooflines[f"decode_b{b}"] = dict(roofline(b, s / k * 1e3, w, k), ms_per_step=round(s / k * 1e3, 4))
+            pt = decode_point(runner, cfg, elt, b, CONTEXT, k, min(args.warmup, 4), peaks)
+            points[f"decode_b{b}"] = pt.pop("tok_s")
+            point_rooflines[f"decode_b{b}"] = pt
         # ---- prefill of one 2,048-token prompt, logits at the last place
         from return_amd.engine import StepEntry
         prompt = [(13 * i + 5) % V for i in range(PREFILL_TOKENS)]
@@ -518,12 +606,7 @@ def main():
             t0 = time.perf_counter()
             one_prefill()
             times.append(time.perf_counter() - t0)
-        pf = min(times[1:])
-        flops = prefill_flops(cfg, PREFILL_TOKENS)
-        prefill = {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS,
-                   "ms": round(pf * 1e3, 3), "frac": round(flops / pf / PEAK_FLOPS[args.dtype], 4),
-                   "measured_peak_TFLOPs": peaks["product_TFLOPs"],
-                   "frac_of_measured": round(flops / pf / (peaks["product_TFLOPs"] * 1e12), 4)}
+        prefill = prefill_record(cfg, args.dtype, PREFILL_TOKENS, min(times[1:]), 1, peaks)
         prefill_kernels = kernel_split(one_prefill, 2)
 
     line = {

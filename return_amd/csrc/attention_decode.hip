@@ -96,27 +96,39 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 // d = 32j + 8g .. +7 of it, the four lanes l, l^16, l^32, l^48 together all of it. The rotary
 // partner of d is d + D/2, which is piece j + D32/2 of the same lane. Sums and products in
 // 32-bit, one rounding to bfloat16 at the end, as in the preparation kernel.
-template <int D32, bool NORM, bool ROPE>
-__device__ __forceinline__ void prepare_head_as(bf16x8_t (&v)[D32], const float* __restrict__ w, float eps,
-                                                const float* __restrict__ cs, const float* __restrict__ sn, int g) {
-    constexpr int D = 32 * D32;
-    // everything this lane needs of the weights and the angles, asked for at once
-    float4_t wv[NORM ? D32 : 1][2], cv[ROPE ? D32 / 2 : 1][2], sv[ROPE ? D32 / 2 : 1][2];
-    if constexpr (NORM) {
+// What a lane needs of the norm weight and of the angles is loaded apart from the arithmetic
+// (HeadWeight, HeadAngles), so that a caller can ask for everything at once and for more after it.
+template <int D32>
+struct HeadWeight {
+    float4_t w[D32][2];
+    __device__ __forceinline__ void load(const float* __restrict__ src, int g) {      // src == nullptr: no norm
+        if (src == nullptr) return;
 #pragma unroll
         for (int j = 0; j < D32; ++j)
 #pragma unroll
-            for (int h = 0; h < 2; ++h) wv[j][h] = *reinterpret_cast<const float4_t*>(w + 32 * j + 8 * g + 4 * h);
+            for (int h = 0; h < 2; ++h) w[j][h] = *reinterpret_cast<const float4_t*>(src + 32 * j + 8 * g + 4 * h);
     }
-    if constexpr (ROPE) {
+};
+
+template <int D32>
+struct HeadAngles {
+    float4_t c[D32 / 2][2], s[D32 / 2][2];
+    __device__ __forceinline__ void load(const float* __restrict__ cs, const float* __restrict__ sn, int g) {
+        if (cs == nullptr) return;                                                     // no rotation
 #pragma unroll
         for (int j = 0; j < D32 / 2; ++j)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                cv[j][h] = *reinterpret_cast<const float4_t*>(cs + 32 * j + 8 * g + 4 * h);
-                sv[j][h] = *reinterpret_cast<const float4_t*>(sn + 32 * j + 8 * g + 4 * h);
+                c[j][h] = *reinterpret_cast<const float4_t*>(cs + 32 * j + 8 * g + 4 * h);
+                s[j][h] = *reinterpret_cast<const float4_t*>(sn + 32 * j + 8 * g + 4 * h);
             }
     }
+};
+
+template <int D32, bool NORM, bool ROPE>
+__device__ __forceinline__ void prepare_head_as(bf16x8_t (&v)[D32], const HeadWeight<D32>& wt, float eps,
+                                                const HeadAngles<D32>& an) {
+    constexpr int D = 32 * D32;
     float rstd = 1.0f;
     if constexpr (NORM) {
         float ss = 0.f;
@@ -151,12 +163,12 @@ __device__ __forceinline__ void prepare_head_as(bf16x8_t (&v)[D32], const float*
             for (int e = 0; e < 4; ++e) {
                 float x1 = a[4 * h + e], x2 = b[4 * h + e];
                 if constexpr (NORM) {
-                    x1 = x1 * rstd * wv[j][h][e];
-                    x2 = x2 * rstd * wv[jp][h][e];
+                    x1 = x1 * rstd * wt.w[j][h][e];
+                    x2 = x2 * rstd * wt.w[jp][h][e];
                 }
                 if constexpr (ROPE) {
-                    const float y1 = x1 * cv[j][h][e] - x2 * sv[j][h][e];
-                    x2 = x2 * cv[j][h][e] + x1 * sv[j][h][e];
+                    const float y1 = x1 * an.c[j][h][e] - x2 * an.s[j][h][e];
+                    x2 = x2 * an.c[j][h][e] + x1 * an.s[j][h][e];
                     x1 = y1;
                 }
                 a[4 * h + e] = x1;
@@ -169,13 +181,13 @@ __device__ __forceinline__ void prepare_head_as(bf16x8_t (&v)[D32], const float*
     }
 }
 
-// w == nullptr: no norm; cs == nullptr: no rotation (the same in every lane)
+// norm: the weight was loaded (its pointer was not null); rope: the angles were (the same in every lane)
 template <int D32>
-__device__ __forceinline__ void prepare_head(bf16x8_t (&v)[D32], const float* __restrict__ w, float eps,
-                                             const float* __restrict__ cs, const float* __restrict__ sn, int g) {
-    if (w != nullptr && cs != nullptr) prepare_head_as<D32, true, true>(v, w, eps, cs, sn, g);
-    else if (w != nullptr) prepare_head_as<D32, true, false>(v, w, eps, cs, sn, g);
-    else if (cs != nullptr) prepare_head_as<D32, false, true>(v, w, eps, cs, sn, g);
+__device__ __forceinline__ void prepare_head(bf16x8_t (&v)[D32], const HeadWeight<D32>& wt, bool norm, float eps,
+                                             const HeadAngles<D32>& an, bool rope) {
+    if (norm && rope) prepare_head_as<D32, true, true>(v, wt, eps, an);
+    else if (norm) prepare_head_as<D32, true, false>(v, wt, eps, an);
+    else if (rope) prepare_head_as<D32, false, true>(v, wt, eps, an);
 }
 
 // LDS of one wave: its value tile, and after its passes its sums for the merge (whichever is larger)
@@ -253,6 +265,25 @@ void attn_decode_kernel(
         return (pt[pi] * Hkv + kvh) * P + (idx - pi * P);     // [page][kv head][row in page]: this head's row
     };
     int row_next = 0;
+    [[maybe_unused]] int first_row = 0;          // FUSED: the rows of the first pass, whose keys are asked for before the loop
+    // the key tiles of a pass, straight into MFMA A operands
+    bf16x8_t ak[4][D32 > 0 ? D32 : 1];
+    bf16x8_t ak_tail[4];
+    auto load_keys = [&](int row) {
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const int r = __shfl(row, st * 16 + n, 64);
+            const bf16* kp = k_pool + (size_t)r * D;
+#pragma unroll
+            for (int j = 0; j < D32; ++j)
+                ak[st][j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
+            if constexpr (TAIL16) {
+                ak_tail[st] = z8;
+                if (g < 2) ak_tail[st] = *reinterpret_cast<const bf16x8_t*>(kp + (D - 16) + 8 * g);
+            }
+        }
+    };
+    const bool any_pass = c_begin <= key_hi && rg.lo <= key_hi;
     if constexpr (FUSED) {
         static_assert(!TAIL16 && D32 % 2 == 0, "the fused preparation needs a head size that is a multiple of 64");
         const size_t width = (size_t)(Hq + 2 * Hkv) * D;
@@ -260,10 +291,33 @@ void attn_decode_kernel(
         const float* cs = fz.cos_t ? fz.cos_t + (size_t)pos_q * (D / 2) : nullptr;
         const float* sn = fz.cos_t ? fz.sin_t + (size_t)pos_q * (D / 2) : nullptr;
         const bf16* qp = tok + (size_t)(h0 + (n < G ? n : 0)) * D;
+        // Everything that waits for no table is asked for at once: q, the norm weights, the angles, and
+        // in the split that holds the new token its k and v. Then the first pass's keys, as soon as the
+        // page table has said where they are: a wave of two passes would otherwise spend a third of its
+        // life on preparing heads before its first key is on its way.
+        HeadWeight<D32> wq, wk;
+        HeadAngles<D32> an;
 #pragma unroll
         for (int j = 0; j < D32; ++j) bq[j] = *reinterpret_cast<const bf16x8_t*>(qp + 32 * j + 8 * g);
-        row_next = row_of(c_begin);                         // asked for together with q, the weights and the angles
-        prepare_head<D32>(bq, fz.w_q, fz.eps, cs, sn, g);
+        row_next = row_of(c_begin);
+        wq.load(fz.w_q, g);
+        an.load(cs, sn, g);
+        bf16x8_t kn[D32];
+        uint4_t vn = {0u, 0u, 0u, 0u};
+        if (has_new) {
+            const bf16* kp = tok + (size_t)(Hq + kvh) * D;
+#pragma unroll
+            for (int j = 0; j < D32; ++j) kn[j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
+            if (lane < LPR) vn = *reinterpret_cast<const uint4_t*>(tok + (size_t)(Hq + Hkv + kvh) * D + lane * 8);
+            wk.load(fz.w_k, g);
+        }
+        if (any_pass) {
+            const int row = row_next;
+            if (c_begin + DEC_CHUNK <= key_hi) row_next = row_of(c_begin + DEC_CHUNK);
+            load_keys(row);
+            first_row = row;
+        }
+        prepare_head<D32>(bq, wq, fz.w_q != nullptr, fz.eps, an, cs != nullptr);
 #pragma unroll
         for (int j = 0; j < D32; ++j) bq[j] = (n < G) ? bq[j] : z8;
         if (has_new) {
@@ -273,13 +327,7 @@ void attn_decode_kernel(
             const int idx = pos_q - start;
             const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
             const size_t row_new = ((size_t)pt[pi] * Hkv + kvh) * P + (idx - pi * P);
-            bf16x8_t kn[D32];
-            const bf16* kp = tok + (size_t)(Hq + kvh) * D;
-#pragma unroll
-            for (int j = 0; j < D32; ++j) kn[j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
-            uint4_t vn = {0u, 0u, 0u, 0u};
-            if (lane < LPR) vn = *reinterpret_cast<const uint4_t*>(tok + (size_t)(Hq + Hkv + kvh) * D + lane * 8);
-            prepare_head<D32>(kn, fz.w_k, fz.eps, cs, sn, g);
+            prepare_head<D32>(kn, wk, fz.w_k != nullptr, fz.eps, an, cs != nullptr);
             if (n == 0) {                                   // one lane of each g holds every piece once
 #pragma unroll
                 for (int j = 0; j < D32; ++j) {
@@ -312,23 +360,13 @@ void attn_decode_kernel(
     for (int dt = 0; dt < D16; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int c0 = c_begin; c0 <= key_hi && rg.lo <= key_hi; c0 += DEC_CHUNK) {
-        const int row = row_next;
-        if (c0 + DEC_CHUNK <= key_hi) row_next = row_of(c0 + DEC_CHUNK);
-
-        // ---- K tiles straight into MFMA A operands
-        bf16x8_t ak[4][D32 > 0 ? D32 : 1];
-        bf16x8_t ak_tail[4];
-#pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            const int r = __shfl(row, st * 16 + n, 64);
-            const bf16* kp = k_pool + (size_t)r * D;
-#pragma unroll
-            for (int j = 0; j < D32; ++j)
-                ak[st][j] = *reinterpret_cast<const bf16x8_t*>(kp + 32 * j + 8 * g);
-            if constexpr (TAIL16) {
-                ak_tail[st] = z8;
-                if (g < 2) ak_tail[st] = *reinterpret_cast<const bf16x8_t*>(kp + (D - 16) + 8 * g);
-            }
+        int row;
+        if (FUSED && c0 == c_begin) {
+            row = first_row;                       // (its keys are on their way already)
+        } else {
+            row = row_next;
+            if (c0 + DEC_CHUNK <= key_hi) row_next = row_of(c0 + DEC_CHUNK);
+            load_keys(row);
         }
         // ---- V rows: 16-byte pieces, all loads of the pass issued now, then into LDS
         uint4_t vv[NVL];
