@@ -284,6 +284,8 @@ void attn_decode_kernel(
         }
     };
     const bool any_pass = c_begin <= key_hi && rg.lo <= key_hi;
+    // (at head size 256 a tile of keys beside everything the preparation holds no longer fits the registers)
+    constexpr bool EARLY_KEYS = FUSED && D16 <= 12;
     if constexpr (FUSED) {
         static_assert(!TAIL16 && D32 % 2 == 0, "the fused preparation needs a head size that is a multiple of 64");
         const size_t width = (size_t)(Hq + 2 * Hkv) * D;
@@ -311,7 +313,7 @@ void attn_decode_kernel(
             if (lane < LPR) vn = *reinterpret_cast<const uint4_t*>(tok + (size_t)(Hq + Hkv + kvh) * D + lane * 8);
             wk.load(fz.w_k, g);
         }
-        if (any_pass) {
+        if (EARLY_KEYS && any_pass) {
             const int row = row_next;
             if (c_begin + DEC_CHUNK <= key_hi) row_next = row_of(c_begin + DEC_CHUNK);
             load_keys(row);
@@ -361,7 +363,7 @@ void attn_decode_kernel(
 
     for (int c0 = c_begin; c0 <= key_hi && rg.lo <= key_hi; c0 += DEC_CHUNK) {
         int row;
-        if (FUSED && c0 == c_begin) {
+        if (EARLY_KEYS && c0 == c_begin) {
             row = first_row;                       // (its keys are on their way already)
         } else {
             row = row_next;

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
     // positions of the first and last row of this wave (wave-uniform, for skipping the mask)
     const int wave_first_pos = pos0 + q_off + wave * QG * 16;
     const int wave_last_pos = wave_first_pos + QG * 16 - 1;
-    float m_run[QG], l_run[QG];
+    float m_run[QG], l_run[QG];                          // (the running maxima are raw scores, before the scale)
     float4_t acc[QG][D16];
 #pragma unroll
     for (int qg = 0; qg < QG; ++qg) {
@@ -240,7 +240,8 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
             }
         }
         MFMA_SETTLE();
-        // Scores in the base-2 domain: s2 = (q.k) * scale * log2(e), so that p = 2^(s2 - m).
+        // p = 2^((s - m) * scale * log2(e)) with s the raw score and m the raw maximum of the row: one fused
+        // multiply-add and one exponential a score (the scale is positive, so the maximum may be taken first).
         // a tile that lies wholly below every row of the wave and inside every window needs no mask
         const bool need_mask = (c0 + BN - 1 > wave_first_pos) || (c0 < first_key) ||
                                (window > 0 && c0 <= wave_last_pos - window);
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
                         const int kpos = c0 + st * 16 + 4 * g + i;
                         bool ok = kpos >= first_key && kpos <= pos_q[qg];
                         if (window > 0) ok = ok && kpos > pos_q[qg] - window;
-                        s[st][i] = ok ? cs[qg][st][i] * scale2 : -INFINITY;
+                        s[st][i] = ok ? cs[qg][st][i] : -INFINITY;
                         mx = fmaxf(mx, s[st][i]);
                     }
                 }
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
                 for (int st = 0; st < BN / 16; ++st) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        s[st][i] = cs[qg][st][i] * scale2;
+                        s[st][i] = cs[qg][st][i];
                         mx = fmaxf(mx, s[st][i]);
                     }
                 }
@@ -275,16 +276,17 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
             const float m_new = fmaxf(m_run[qg], mx);
             // a row that sees no key yet (all of this pass lies above it or outside its window) keeps m = -inf
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float off = -m_use * scale2;
             float lsum = 0.f;
 #pragma unroll
             for (int st = 0; st < BN / 16; ++st)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    s[st][i] = __builtin_amdgcn_exp2f(s[st][i] - m_use);      // 2^(-inf) = 0 for masked keys
+                    s[st][i] = __builtin_amdgcn_exp2f(fmaf(s[st][i], scale2, off));      // 2^(-inf) = 0 for masked keys
                     lsum += s[st][i];
                 }
             lsum = rows_sum(lsum);
-            const float alpha = (m_run[qg] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qg] - m_use);
+            const float alpha = (m_run[qg] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run[qg] - m_use) * scale2);
             l_run[qg] = l_run[qg] * alpha + lsum;
             if (__any(m_new != m_run[qg])) {             // some row's maximum moved: rescale what is summed so far
 #pragma unroll
@@ -349,9 +351,9 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
         for (int qg = 0; qg < QG; ++qg) {
             const float* mq = ms + qg * MERGE_SLOTS * 64;
             const float m1 = mq[0], l1 = mq[64];
-            const float m = fmaxf(m_run[qg], m1);
-            const float a0 = (m_run[qg] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[qg] - m);
-            const float a1 = (m1 == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+            const float m = fmaxf(m_run[qg], m1);        // (raw scores: the scale comes in with the exponent)
+            const float a0 = (m_run[qg] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run[qg] - m) * scale2);
+            const float a1 = (m1 == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m1 - m) * scale2);
             l_run[qg] = l_run[qg] * a0 + l1 * a1;
 #pragma unroll
             for (int dt = 0; dt < D16; ++dt)

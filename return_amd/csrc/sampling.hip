@@ -9,7 +9,9 @@
 //
 // The draw uses a uniform number u in [0,1) that the host supplies per row: the token is the
 // first, in vocabulary order, at which the running sum of kept probabilities exceeds u.
-// Tokens that tie with the k-th value, or with the top-p boundary value, are all kept.
+// Among tokens that tie at a boundary the earlier ones in the vocabulary stay, as a stable sort
+// puts them first: exactly top_k tokens are kept (rollout/model.py:45-50 keeps topk(k)), and of the
+// tokens that tie with the top-p boundary value those before which at most top_p of the mass lies.
 //
 // top-k and top-p need a threshold among the largest logits. The row's tokens within CAND_SPAN of
 // the largest logit (in units of the temperature: every other token weighs less than e^-16 of the
@@ -30,6 +32,10 @@
 __device__ __forceinline__ uint32_t order_key(float f) {
     const uint32_t b = __float_as_uint(f);
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);      // ascending float order -> ascending uint
+}
+
+__device__ __forceinline__ float key_value(uint32_t k) {      // the float whose order_key is k
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
 // f(i, v) for every element of the row, four at a time where the row allows 16-byte loads
@@ -91,9 +97,10 @@ __device__ __forceinline__ fixed_t block_sum_fixed(fixed_t v, fixed_t* wsum) {
 // A range of 2^32 keys takes three passes. wsum: CAND_WAVES words, sh_b, sh_above: one word each, all LDS.
 #define SEARCH_BITS 11
 #define SEARCH_BUCKETS (1 << SEARCH_BITS)
+// above (may be nullptr) is told measure{key > t}.
 template <typename Visit>
 __device__ uint32_t search_threshold(Visit visit, int tid, uint32_t lo, uint32_t hi, fixed_t limit, fixed_t* fx,
-                                     fixed_t* wsum, int* sh_b, fixed_t* sh_above) {
+                                     fixed_t* wsum, int* sh_b, fixed_t* sh_above, fixed_t* above = nullptr) {
     static_assert(SEARCH_BUCKETS == 2 * SAMPLE_THREADS, "a thread looks after two runs");
     const int wave = tid >> 6, lane = tid & 63;
     fixed_t above_hi = 0ull;
@@ -137,7 +144,33 @@ __device__ uint32_t search_threshold(Visit visit, int tid, uint32_t lo, uint32_t
         hi = new_hi;
         __syncthreads();
     }
+    if (above) *above = above_hi;
     return lo;
+}
+
+// Of the tokens that tie at a boundary, the first `stay` in vocabulary order stay: returns the index of the
+// last of them (`upto` if all of them stay). count_ties(f) calls f(index) for every tying token of this thread
+// with index <= upto. One pass counts them; only if they are more than may stay, the index is searched.
+// (A function of its own, not inlined: it runs four times in the kernel, and inlined the kernel no longer
+// fits the 128 registers that a block of 1,024 threads leaves a lane.)
+template <typename Ties>
+__device__ __noinline__ int tie_cut(Ties ties, int tid, int V, unsigned long long stay, int upto, fixed_t* fx, fixed_t* wsum,
+                       int* sh_b, fixed_t* sh_above) {
+    fixed_t mine = 0ull;
+    ties([&](int) { mine += 1ull; });
+    const fixed_t n = block_sum_fixed(mine, wsum);
+    if (stay >= n) return upto;
+    if (stay == 0ull) return -1;
+    // the stay-th tie from the front: the smallest t with at most stay - 1 ties at keys V - 1 - index above it
+    const uint32_t t = search_threshold(
+        [&](uint32_t lo, uint32_t hi, auto add) {
+            ties([&](int i) {
+                const uint32_t key = (uint32_t)(V - 1 - i);
+                if (key > lo && key <= hi) add(key, 1ull << 40);
+            });
+        },
+        tid, 0u, (uint32_t)(V - 1), (fixed_t)(stay - 1ull) << 40, fx, wsum, sh_b, sh_above);
+    return V - 1 - (int)t;
 }
 
 // The draw's first step: wmass[w] is the kept mass of wave w's run of tokens (runs in vocabulary order).
@@ -261,7 +294,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const int k = top_k[row];
     const float p = top_p[row];
     const bool want_k = k > 0 && k < V, want_p = p < 1.0f;
-    uint32_t keep_key = 0u;                   // keep tokens whose key >= keep_key
+    // what stays: tokens whose key is above keep_key, and of those whose key is keep_key the ones up to tie_limit
+    uint32_t keep_key = 0u;
+    int tie_limit = 0x7fffffff;
+    auto kept = [&](uint32_t key, int i) { return key > keep_key || (key == keep_key && i <= tie_limit); };
 
     if (want_k || want_p) {
         // ---- the list: wave w goes through its run of the row, 64 tokens a load, and appends the tokens
@@ -328,7 +364,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             // a thread's entries for the searches: place (tid % CAND_PER_WAVE) of every other wave's part
             if (listed) {
                 uint32_t key[CAND_OWN];
-                fixed_t weight[CAND_OWN];
+                float weight[CAND_OWN];                    // exp((x - max) / T), made a whole number where it is added
+                int idx[CAND_OWN];                         // the entry's token; -1: no entry
                 const int half = tid / CAND_PER_WAVE, off = tid - half * CAND_PER_WAVE;
 #pragma unroll
                 for (int e = 0; e < CAND_OWN; ++e) {
@@ -336,33 +373,57 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                     const bool there = off < cnt[w];
                     const float v = there ? cv[w * CAND_PER_WAVE + off] : 0.f;
                     key[e] = there ? order_key(v) : 0u;
-                    weight[e] = there ? to_fixed(__expf((v - gmax) * inv_t)) : 0ull;
+                    weight[e] = there ? __expf((v - gmax) * inv_t) : 0.f;
+                    idx[e] = there ? ci[w * CAND_PER_WAVE + off] : -1;
                 }
+                // the entries that tie at key t, up to token `upto`
+                auto ties_at = [&](uint32_t t, int upto) {
+                    return [&key, &idx, t, upto](auto f) {
+#pragma unroll
+                        for (int e = 0; e < CAND_OWN; ++e)
+                            if (idx[e] >= 0 && key[e] == t && idx[e] <= upto) f(idx[e]);
+                    };
+                };
                 // top-k: the k-th largest is on the list; below cut_key - 1 nothing of it lies
-                if (want_k)
+                if (want_k) {
+                    fixed_t above = 0ull;
                     keep_key = search_threshold(
                         [&](uint32_t lo, uint32_t hi, auto add) {
 #pragma unroll
                             for (int e = 0; e < CAND_OWN; ++e)
                                 if (key[e] > lo && key[e] <= hi) add(key[e], 1ull << 40);
                         },
-                        tid, cut_key - 1u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above);
+                        tid, cut_key - 1u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above, &above);
+                    // of the tokens that tie with the k-th value, as many stay as make k with those above them
+                    tie_limit = tie_cut(ties_at(keep_key, 0x7fffffff), tid, V, (unsigned long long)k - (above >> 40),
+                                        0x7fffffff, fx, wsum, &sh_b, &sh_above);
+                }
                 if (want_p) {
                     fixed_t zc = 0ull;
 #pragma unroll
-                    for (int e = 0; e < CAND_OWN; ++e) zc += key[e] >= keep_key && key[e] != 0u ? weight[e] : 0ull;
+                    for (int e = 0; e < CAND_OWN; ++e) zc += idx[e] >= 0 && kept(key[e], idx[e]) ? to_fixed(weight[e]) : 0ull;
                     zc = block_sum_fixed(zc, wsum);
                     const fixed_t z = zc + (fixed_t)((double)z_rest * (double)FIXED_ONE_F);
                     const fixed_t limit = (fixed_t)((double)p * (double)z);
                     // the boundary is on the list if the list's mass is more than p of the whole (always, after top-k)
                     if (want_k || zc > limit) {
+                        const uint32_t k_key = keep_key;     // what top-k left: the search goes over that
+                        const int k_limit = tie_limit;
+                        fixed_t above = 0ull;
                         keep_key = search_threshold(
                             [&](uint32_t lo, uint32_t hi, auto add) {
 #pragma unroll
                                 for (int e = 0; e < CAND_OWN; ++e)
-                                    if (key[e] > lo && key[e] <= hi) add(key[e], weight[e]);
+                                    if (idx[e] >= 0 && key[e] > lo && key[e] <= hi &&
+                                        (key[e] > k_key || idx[e] <= k_limit)) add(key[e], to_fixed(weight[e]));
                             },
-                            tid, want_k ? keep_key : cut_key - 1u, top_key, limit, fx, wsum, &sh_b, &sh_above);
+                            tid, want_k ? k_key : cut_key - 1u, top_key, limit, fx, wsum, &sh_b, &sh_above, &above);
+                        // of the tokens that tie with the boundary value, the i-th in vocabulary order stays while
+                        // what lies before it, the mass above them and i of their own, is at most top_p of the whole
+                        const fixed_t each = to_fixed(__expf((key_value(keep_key) - gmax) * inv_t));
+                        const unsigned long long stay = each ? (limit - above) / each + 1ull : ~0ull;
+                        const int upto = keep_key == k_key ? k_limit : 0x7fffffff;
+                        tie_limit = tie_cut(ties_at(keep_key, upto), tid, V, stay, upto, fx, wsum, &sh_b, &sh_above);
                     } else {
                         listed = false;
                     }
@@ -376,7 +437,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                 float mine = 0.f;
                 for (int o = o0; o < o1; ++o) {
                     const float v = cv[wave * CAND_PER_WAVE + o];
-                    if (order_key(v) >= keep_key) mine += __expf((v - gmax) * inv_t);
+                    if (kept(order_key(v), ci[wave * CAND_PER_WAVE + o])) mine += __expf((v - gmax) * inv_t);
                 }
                 const float upto = wave_running_sum(mine, lane);
                 __syncthreads();
@@ -403,7 +464,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                     int tok = argmax;
                     for (int o = o0; o < o1; ++o) {
                         const float v = cv[wave * CAND_PER_WAVE + o];
-                        if (order_key(v) >= keep_key) {
+                        if (kept(order_key(v), ci[wave * CAND_PER_WAVE + o])) {
                             tok = ci[wave * CAND_PER_WAVE + o];      // the last kept entry if the target is never passed
                             run += __expf((v - gmax) * inv_t);
                             if (run > target) break;
@@ -418,10 +479,20 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
         __syncthreads();
         keep_key = 0u;
+        tie_limit = 0x7fffffff;
+        // the row's tokens that tie at key t, up to token `upto`
+        auto ties_at = [&](uint32_t t, int upto) {
+            return [x, V, tid, t, upto](auto f) {
+                for_each_logit(x, V, tid, [&](int i, float v) {
+                    if (order_key(v) == t && i <= upto) f(i);
+                });
+            };
+        };
 
         // ---- over the whole row. top-k: the key of the k-th largest value is the smallest key with at most
         // k - 1 tokens above it
-        if (want_k)
+        if (want_k) {
+            fixed_t above = 0ull;
             keep_key = search_threshold(
                 [&](uint32_t lo, uint32_t hi, auto add) {
                     for_each_logit(x, V, tid, [&](int, float v) {
@@ -429,22 +500,34 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                         if (key > lo && key <= hi) add(key, 1ull << 40);
                     });
                 },
-                tid, 0u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above);
+                tid, 0u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above, &above);
+            tie_limit = tie_cut(ties_at(keep_key, 0x7fffffff), tid, V, (unsigned long long)k - (above >> 40),
+                                0x7fffffff, fx, wsum, &sh_b, &sh_above);
+        }
         // top-p: the smallest key with at most p of the kept mass above it
         if (want_p) {
             fixed_t z = 0ull;
-            for_each_logit(x, V, tid, [&](int, float v) {
-                if (order_key(v) >= keep_key) z += to_fixed(__expf((v - gmax) * inv_t));
+            for_each_logit(x, V, tid, [&](int i, float v) {
+                if (kept(order_key(v), i)) z += to_fixed(__expf((v - gmax) * inv_t));
             });
             z = block_sum_fixed(z, wsum);
+            const fixed_t limit = (fixed_t)((double)p * (double)z);
+            const uint32_t k_key = keep_key;             // what top-k left: the search goes over that
+            const int k_limit = tie_limit;
+            fixed_t above = 0ull;
             keep_key = search_threshold(
                 [&](uint32_t lo, uint32_t hi, auto add) {
-                    for_each_logit(x, V, tid, [&](int, float v) {
+                    for_each_logit(x, V, tid, [&](int i, float v) {
                         const uint32_t key = order_key(v);
-                        if (key > lo && key <= hi) add(key, to_fixed(__expf((v - gmax) * inv_t)));
+                        if (key > lo && key <= hi && (key > k_key || i <= k_limit))
+                            add(key, to_fixed(__expf((v - gmax) * inv_t)));
                     });
                 },
-                tid, keep_key, top_key, (fixed_t)((double)p * (double)z), fx, wsum, &sh_b, &sh_above);
+                tid, k_key, top_key, limit, fx, wsum, &sh_b, &sh_above, &above);
+            const fixed_t each = to_fixed(__expf((key_value(keep_key) - gmax) * inv_t));
+            const unsigned long long stay = each ? (limit - above) / each + 1ull : ~0ull;
+            const int upto = keep_key == k_key ? k_limit : 0x7fffffff;
+            tie_limit = tie_cut(ties_at(keep_key, upto), tid, V, stay, upto, fx, wsum, &sh_b, &sh_above);
         }
     }
 
@@ -454,7 +537,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     // the block in which it does, and goes through that block again, token by token.
     {
         auto kept_mass = [&](int i, float v) {             // (a token beyond the run's end has none: exp(-inf))
-            return (i < end && order_key(v) >= keep_key) ? __expf((v - gmax) * inv_t) : 0.f;
+            return (i < end && kept(order_key(v), i)) ? __expf((v - gmax) * inv_t) : 0.f;
         };
         __shared__ float bmass[CAND_WAVES][SAMPLE_BLOCKS];
         const int n_it = (end - beg + 255) / 256;            // this wave's blocks
@@ -518,7 +601,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                 int first = -1;
 #pragma unroll
                 for (int c = 3; c >= 0; --c) {
-                    const bool is_kept = i + c < end && order_key(a[j][c]) >= keep_key;
+                    const bool is_kept = i + c < end && kept(order_key(a[j][c]), i + c);
                     if (is_kept && base + s[c] > target) first = c;
                     if (is_kept) last_kept = max(last_kept, i + c);
                 }

@@ -61,6 +61,11 @@ class StepBatch:
     decode_segs: Optional[torch.Tensor] = None     # int32 [n_decode] request numbers; None: all of them
     max_decode_seq_len: int = 0
     decode_len_is_bound: bool = False              # max_decode_seq_len is an upper bound (a graph's bucket), not the longest length
+    # (requests, longest length) that the kernel set bases its choice of splits on, when these are not the step's
+    # own: the runner names a decode step's class (the batch size and context bucket of the graph that serves or
+    # would serve it), so that a step run eagerly and the same step replayed from a graph take the same splits
+    # and with them the same order of sums
+    decode_rule: Optional[tuple] = None
     n_prefill_tokens: int = 0
     prefill_toks: Optional[torch.Tensor] = None    # int32 token rows of the others; None: all rows
     prefill_segs: List[int] = dataclasses.field(default_factory=list)   # host: their request numbers

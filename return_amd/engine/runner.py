@@ -294,16 +294,17 @@ class ModelRunner:
         graphs = self.engine_config.use_graphs and self.rt.device.type == "cuda"
         rows = self.graph_batch_size(n) if graphs else n
         pad = rows - n
-        if graphs:
-            key = self._graph_key(rows, max(self.cache.seq_len(rid) for rid in request_ids) + 1)
-            if key not in self._graphs:
-                self._capture(key)
+        # the step's class: what a graph for it is keyed by, with or without graphs
+        key = self._graph_key(self.graph_batch_size(n), max(self.cache.seq_len(rid) for rid in request_ids) + 1)
+        if graphs and key not in self._graphs:
+            self._capture(key)
         tables = self.cache.begin_step([(rid, 1) for rid in request_ids])
         try:
             tables = self.cache.pad_tables(tables, pad)
             host_tokens = [[0]] * rows if tokens is None else [[int(t)] for t in tokens] + [[0]] * pad
             batch = self.builder.build(tables, host_tokens, list(range(rows)),
                                        self._flat_columns(list(columns) + [None] * pad, tables) if columns else None)
+            batch.decode_rule = key
             if tokens is None:
                 # after the tables' copy and before the step: the sampled tokens become the new tokens
                 if self._samp_copied is not None:
@@ -368,6 +369,7 @@ class ModelRunner:
             batch = self.builder.build(tables, [[0]] * rows, list(range(rows)))
             batch.max_decode_seq_len = bucket
             batch.decode_len_is_bound = True
+            batch.decode_rule = key
             with torch.no_grad():
                 side = torch.cuda.Stream(dev)
                 side.wait_stream(torch.cuda.current_stream(dev))

@@ -819,10 +819,14 @@ class HipOps:
         slower otherwise (batch 40, 48, 72: 5 to 15 %): a workgroup of eight waves fills a CU's LDS, and
         a last round that is far from full leaves most of the chip idle."""
         longest = step.max_decode_seq_len
+        # what the choice is based on: the step's own numbers, or the class its runner names (then a step run
+        # eagerly and its replay from a graph choose alike and sum in the same order)
+        rule = getattr(step, "decode_rule", None)
+        n_rule, l_rule = rule if rule else (step.n_decode, longest)
         S = self.decode_split_tokens
-        groups = step.n_decode * n_kv * -(-(n_q // n_kv) // 16)
+        groups = n_rule * n_kv * -(-(n_q // n_kv) // 16)
         waves = self.lib.ra_attention_decode_merge_waves(D)
-        if S <= 0 and window == 0 and waves >= 2 and longest > 64 and self.decode_merge_round > 0 \
+        if S <= 0 and window == 0 and waves >= 2 and l_rule > 64 and self.decode_merge_round > 0 \
                 and (groups % self.decode_merge_round == 0 or groups >= 3 * self.decode_merge_round):
             # (the kernel cuts every request into W even splits of its own length)
             # Waves of such a workgroup (measured, 8 kv heads of 128, batch 32 to 128, contexts of 2,048 and
@@ -831,18 +835,21 @@ class HipOps:
             # up to 4,096 (and 2 % slower with longer, uneven ones), four up to 5 % faster below two rounds.
             want = self.decode_merge_waves
             if want <= 0:
-                want = 4 if groups < 2 * self.decode_merge_round else (2 if longest <= 4096 else 8)
-            W = min(want, waves, -(-longest // 64))
+                want = 4 if groups < 2 * self.decode_merge_round else (2 if l_rule <= 4096 else 8)
+            W = min(want, waves, -(-l_rule // 64))
             return 64, max(W, 2), True
         if S <= 0:
             # about two thousand waves in all (eight per CU) fill the chip; fewer, longer
             # splits spend less on starting up and on the merge (measured from 1 to 128 requests)
-            chunks = step.n_decode * n_kv * ((longest + 63) // 64)
-            S = 64 * max(2, -(-chunks // 2048), -(-longest // 4096))     # and at most 64 splits a request
-            if getattr(step, "decode_len_is_bound", False):
-                # the lengths lie somewhere below `longest` (a graph's context bucket): splits
+            # (a few hundred waves do not fill it: then a wave takes one pass of 64 keys and all of a
+            # request's loads are on their way at once; batch 1 over 2,048 keys 10.0 against 10.8 µs, batch 2
+            # 11.8 against 12.4, from about a thousand waves on 15.4 against 14.8)
+            chunks = n_rule * n_kv * ((l_rule + 63) // 64)
+            S = 64 * max(1 if chunks <= 640 else 2, -(-chunks // 2048), -(-l_rule // 4096))     # and at most 64 splits a request
+            if rule or getattr(step, "decode_len_is_bound", False):
+                # the lengths lie somewhere below the bound (a graph's context bucket): splits
                 # of at most an eighth of it keep the work of a request even
-                S = min(S, max(128, longest // 8 // 64 * 64))
+                S = min(S, max(128 if S > 64 else 64, l_rule // 8 // 64 * 64))
         max_splits = (longest - 1) // S + 1
         if window > 0:                       # a window spans at most this many splits
             max_splits = min(max_splits, (window + S - 2) // S + 1)

@@ -854,8 +854,7 @@ def test_sample_matches_plain_draw(ops, ref, V):
 def test_sample_at_the_full_vocabulary(ops):
     """top-k and top-p at a vocabulary of 151,936 (the threshold search over the whole row, pass by
     pass): every row's token is where the plain distribution's running sum, in vocabulary order,
-    passes the row's uniform number; peaked and flat rows, ties above the boundary (tokens that tie
-    with the boundary value itself are all kept here, one by one in the plain rule), k = 1, p near 0."""
+    passes the row's uniform number; peaked and flat rows, ties above the boundary, k = 1, p near 0."""
     from tests.plain import qwen3_plain as plain
     V, M = 151936, 32
     logits = rnd(M, V, seed=73, scale=3.0)
@@ -877,6 +876,45 @@ def test_sample_at_the_full_vocabulary(ops):
         assert before - 1e-4 <= float(u[r]) <= float(c[tok]) + 1e-4, (r, tok, before, float(u[r]), float(c[tok]))
         lp = out[r, 1:2].contiguous().view(torch.float32)
         assert abs(float(lp) - plain.chosen_logprob(logits[r].cpu(), tok)) < 1e-3
+
+
+@pytest.mark.parametrize("V,path", [(1000, 1), (20001, 2), (151936, 2)])
+def test_sample_cuts_ties_at_a_boundary_in_vocabulary_order(ops, ref, V, path):
+    """Logits from a handful of values, so that hundreds of tokens tie at every boundary: exactly top_k
+    tokens stay (rollout/model.py:45-50 keeps topk(k)), of the tying ones the first in the vocabulary, as the
+    plain rule's stable sort has them; of the tokens that tie at the top-p boundary those before which at most
+    top_p of the mass lies (the crossing token stays, rollout/model.py:51-55). Every row's token is the plain
+    draw's, from the list of the largest logits (a vocabulary that fits it) and from the whole row."""
+    M = 64
+    g = torch.Generator().manual_seed(V)
+    logits = torch.randint(0, 5, (M, V), generator=g).float()
+    logits[:, 7] = 5.0                                            # one largest, so that the rows are not flat at the top
+    logits = logits.to(DEV)
+    u = torch.rand(M, generator=g).to(DEV)
+    temp = torch.tensor([1.0, 0.7, 1.5, 1.0] * (M // 4), device=DEV)
+    top_k = torch.tensor([50, 0, 333, 2, 0, 1000, 7, 0] * (M // 8), dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([1.0, 0.3, 0.9, 1.0, 0.05, 0.5, 0.6, 0.999] * (M // 8), device=DEV)
+    way = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+    a = ops.sample(logits, temp, top_k, top_p, u, path=way)
+    b = ref.sample(logits, temp, top_k, top_p, u)
+    assert a[:, 0].tolist() == b[:, 0].tolist()
+    assert set(way.tolist()) == {path}
+    # and the kept set itself, row by row: a sweep of uniform numbers draws exactly the plain rule's tokens
+    from tests.plain import qwen3_plain as plain
+    for r in (0, 1, 3, 6):
+        d = plain.sample_distribution(logits[r].cpu(), float(temp[r]), int(top_k[r]), float(top_p[r]))
+        support = set(d.nonzero().flatten().tolist())
+        n = 2048
+        sweep = ((torch.arange(n) + 0.5) / n).to(DEV)
+        rows = logits[r:r + 1].expand(n, V).contiguous()
+        out = ops.sample(rows, temp[r:r + 1].expand(n).contiguous(), top_k[r:r + 1].expand(n).contiguous(),
+                         top_p[r:r + 1].expand(n).contiguous(), sweep)
+        drawn = set(out[:, 0].tolist())
+        assert drawn <= support, f"row {r}: tokens outside the kept set were drawn: {sorted(drawn - support)[:5]}"
+        if len(support) <= 64:
+            assert drawn == support, f"row {r}: kept tokens that no uniform number reaches: {sorted(support - drawn)[:5]}"
+        if int(top_k[r]) > 0 and float(top_p[r]) >= 1.0:
+            assert len(support) == int(top_k[r])
 
 
 def test_sample_from_the_list_of_the_largest_logits_and_from_the_whole_row(ops):
