@@ -168,6 +168,9 @@ def measured_peaks(runner, dtype):
     return out
 
 
+PROFILE_KERNELS = True      # --no-kernels: no profiler pass of bench.py's own (for runs under another profiler)
+
+
 def kernel_split(run, steps):
     """Device time of `steps` calls of run() by kernel, from a profiler pass of its own (outside every
     timed region; what rollout/utils/prof_graph.py:64-101 does for the reference's decode): the ten
@@ -175,11 +178,17 @@ def kernel_split(run, steps):
     import re
     import torch
     from torch.profiler import ProfilerActivity, profile
+    if not PROFILE_KERNELS:
+        return {"skipped": "--no-kernels"}
     try:
         with profile(activities=[ProfilerActivity.CUDA]) as prof:
             for _ in range(steps):
                 run()
             torch.cuda.synchronize()
+            # (the tracer hands over its last records late: without a pause the step's last kernels are missing)
+            torch.zeros(1, device="cuda:0").add_(1)
+            torch.cuda.synchronize()
+            time.sleep(0.2)
         per = {}
         for e in prof.key_averages():
             us = getattr(e, "self_device_time_total", 0) or getattr(e, "self_cuda_time_total", 0)
@@ -270,16 +279,21 @@ def shape_of(cfg, **more):
 
 def continuous_4b(args):
     """Continuous batching on the Qwen3-4B shape: 128 requests, prompts of 64 to 4,096 tokens and
-    32 to 512 new tokens each (uniform), prompts in portions of 512 beside the decoded tokens,
-    through Engine.generate. value: generated tokens a second over the whole run."""
+    32 to 512 new tokens each (uniform), prompts in portions of 512 beside the decoded tokens (up to
+    --step-tokens tokens a step), as Engine.generate runs them. value: generated tokens a second over
+    the whole run."""
     import random
     import torch
     from return_amd import SamplingParams
     from return_amd.engine import Engine
     n = args.batch if args.batch != 8 else 128
+    # A step's token budget: every decoding request's token and up to four portions of 512 prompt tokens. What
+    # a step costs whatever it brings (the weights read once, the decode attention of every live request) is
+    # shared by more prompt tokens then: one portion a step gives 3,840 generated tok/s, four 4,660, sixteen 4,860.
+    budget = args.step_tokens or 2048 + n
     cfg, runner = build_runner(0, args.dtype, n, raw=QWEN3_4B, use_graphs=not args.no_graphs,
                                tune_products=not args.no_tune, defer_norms=not args.no_defer_norms,
-                               max_token=n * 4608, max_step_tokens=512 + n, prefill_chunk=512)
+                               max_token=n * 4608, max_step_tokens=budget, prefill_chunk=512)
     elt = 2 if args.dtype == "bfloat16" else 4
     peaks = measured_peaks(runner, args.dtype)
     eng = Engine(runner=runner)
@@ -324,7 +338,7 @@ def continuous_4b(args):
             "ms_per_step": round(secs / eng.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
             "config": shape_of(cfg, model="Qwen3-4B shape", global_batch=n, prompt_tokens=read, new_tokens=made,
-                               prefill_chunk=512, max_context=4608, hip_graphs=not args.no_graphs,
+                               prefill_chunk=512, step_tokens=budget, max_context=4608, hip_graphs=not args.no_graphs,
                                weights="random N(0,0.02)"),
             "seconds": round(secs, 3), "measured": peaks,
             # the whole run as matrix work: prompt and generated tokens through every projection
@@ -537,10 +551,16 @@ def main():
     ap.add_argument("--page-size", type=int, default=PAGE, help=f"tokens per cache page (the benchmark's is {PAGE})")
     ap.add_argument("--no-defer-norms", action="store_true",
                     help="run every RMSNorm as a kernel of its own instead of inside the products around it")
+    ap.add_argument("--step-tokens", type=int, default=0,
+                    help="continuous_4b: token budget of a step (default: 2,048 prompt tokens beside one token of every request)")
+    ap.add_argument("--no-kernels", action="store_true",
+                    help="leave out the profiler passes that split a step's time by kernel (for runs under rocprofv3)")
     ap.add_argument("--no-tune", action="store_true",
                     help="choose the kernel of every projection by rule instead of measuring at load "
                          "(keeps the measuring launches out of a profile)")
     args = ap.parse_args()
+    global PROFILE_KERNELS
+    PROFILE_KERNELS = not args.no_kernels
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2

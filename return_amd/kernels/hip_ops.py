@@ -117,6 +117,8 @@ class HipOps:
         self.decode_merge_waves = 0          # waves of such a workgroup; 0: by the number of pairs and the context
         self.prefill_key_split = 0           # groups of waves that share a q tile's keys (1 or 2); 0: by the number of tiles
         self.prefill_small_tiles = True      # q tiles of 64 rows instead of 128 while those would not fill the chip
+        self.overlap_attention = True        # mixed steps: the decode and the prefill attention side by side on two streams
+        self._side_stream = None
         self.skinny_max_grid = 0             # 0: one workgroup per 16 weight rows
         self.gated_skinny_rows = 8           # up to this many rows gate-up and SiLU-mul are one kernel
         self.own_gemm = False                # True: bf16 products of many rows use the hand-written MFMA kernel
@@ -697,22 +699,48 @@ class HipOps:
                 h = torch.zeros(rows, N, device=self.device, dtype=torch.float32)
                 wn = torch.ones(N, device=self.device, dtype=torch.float32)
                 normed = torch.empty(rows, N, device=self.device, dtype=torch.bfloat16)
-            times = {}
+            runs = {}
             for how in cands:
                 if gated:
-                    run = lambda w, how=how: self._gated_by(how, x, w)
+                    runs[how] = lambda w, how=how: self._gated_by(how, x, w)
                 elif how.startswith("split"):
-                    run = lambda w, how=how: self.add_rmsnorm(h, self._split_product(x, w, int(how[5:])), wn, 1e-6, normed)
+                    runs[how] = lambda w, how=how: self.add_rmsnorm(h, self._split_product(x, w, int(how[5:])), wn, 1e-6, normed)
                 elif out_dtype == "residual":
-                    run = lambda w, how=how: self.add_rmsnorm(h, self._linear_by(how, x, w, torch.bfloat16), wn, 1e-6, normed)
+                    runs[how] = lambda w, how=how: self.add_rmsnorm(h, self._linear_by(how, x, w, torch.bfloat16), wn, 1e-6, normed)
                 else:
-                    run = lambda w, how=how: self._linear_by(how, x, w, out_dtype)
-                times[how] = self._time_over(run, weights, launches)
+                    runs[how] = lambda w, how=how: self._linear_by(how, x, w, out_dtype)
+            times = self._time_ways(runs, weights, launches)
         finally:
             self.product_plan = saved
         self._times[key] = dict(times)
         best = min(times, key=times.get)
         return best if best != rule and times[best] < margin * times[rule] else None
+
+    def _time_ways(self, runs, weights, launches, rounds=3):
+        """Seconds per call of every way in ``runs`` (name -> run(w)), the weights taken in turn: one captured
+        graph per way, and the ways timed in turn, round after round, each way's fastest round counting. So a
+        clock that is still rising, or falls under load, meets every way alike, and the choice between two
+        ways that are close does not follow the order in which they were measured."""
+        import time
+        graphs = {}
+        for how, run in runs.items():
+            run(weights[0])
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(launches):
+                    run(weights[i % len(weights)])
+            graph.replay()
+            graphs[how] = graph
+        torch.cuda.synchronize(self.device)
+        best = {how: float("inf") for how in runs}
+        for _ in range(rounds):
+            for how, graph in graphs.items():
+                t0 = time.perf_counter()
+                graph.replay()
+                torch.cuda.synchronize(self.device)
+                best[how] = min(best[how], time.perf_counter() - t0)
+        return {how: t / launches for how, t in best.items()}
 
     def _time_over(self, run, weights, launches):
         """Seconds per call of run(w), the weights taken in turn, launched from one captured graph."""
@@ -769,7 +797,10 @@ class HipOps:
         window = int(window)
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
         fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
-        if fast_decode:
+        fast_prefill = q.dtype == torch.bfloat16 and bool(step.prefill_tiles) and D % 16 == 0 and D <= 256 and \
+            (fast_decode or step.n_decode == 0)
+
+        def decode_part():
             S, max_splits, merge = self._decode_splits(step, n_q, n_kv, D, window)
             nd = step.n_decode
             part_acc = part_ml = None
@@ -780,13 +811,8 @@ class HipOps:
                 _ptr(q), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(k_pool), _ptr(v_pool), *tabs,
                 _ptr(step.decode_segs), nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
                 1 if merge else 0, self._stream()), "attention_decode_bf16")
-            if step.n_prefill_tokens == 0:
-                return
-            toks, n_tok = step.prefill_toks, step.n_prefill_tokens
-        else:
-            toks, n_tok = None, T
-        if q.dtype == torch.bfloat16 and step.prefill_tiles and D % 16 == 0 and D <= 256 and \
-                (fast_decode or step.n_decode == 0):
+
+        def prefill_part():
             rows = self.lib.ra_attention_prefill_tile_rows(D)
             tiles = step.prefill_tiles.get(rows)
             if tiles is None:
@@ -805,6 +831,35 @@ class HipOps:
                 _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], rows,
                 split, n_q, n_kv, D, P, float(scale), window, self._stream()),
                 "attention_prefill_bf16")
+
+        if fast_decode and fast_prefill and step.n_prefill_tokens > 0:
+            # A step of prompt portions beside decoded tokens: the two kernels work on different rows of q and
+            # out, one is bound by memory and the other by the matrix cores and the latency inside its waves,
+            # so they run side by side on two streams (never while a graph is being captured: such steps are
+            # not captured anyway, and a fork and join inside a graph costs more than it gives).
+            if self.overlap_attention and not torch.cuda.is_current_stream_capturing():
+                main = torch.cuda.current_stream(self.device)
+                if self._side_stream is None:
+                    self._side_stream = torch.cuda.Stream(self.device)      # (default priority, like every stream here)
+                side = self._side_stream
+                side.wait_stream(main)               # q and the new keys and values are written
+                with torch.cuda.stream(side):
+                    prefill_part()
+                decode_part()
+                main.wait_stream(side)               # what follows reads both kernels' rows of out
+            else:
+                decode_part()
+                prefill_part()
+            return
+        if fast_decode:
+            decode_part()
+            if step.n_prefill_tokens == 0:
+                return
+            toks, n_tok = step.prefill_toks, step.n_prefill_tokens
+        else:
+            toks, n_tok = None, T
+        if fast_prefill:
+            prefill_part()
             return
         self._check(self.lib.ra_attention_plain(
             _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,

@@ -445,7 +445,7 @@ def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
         assert (ops.route_gated(rows, N, K) if gated else ops.route_linear(rows, N, K, out_dtype)) == how
     before = dict(plan)
     calls = []
-    monkeypatch.setattr(ops, "_time_over", lambda *a: calls.append(a) or 1.0)
+    monkeypatch.setattr(ops, "_time_ways", lambda runs, *a: calls.append(a) or {how: 1.0 for how in runs})
     plan.clear()
     ops.tune_products(products, max_rows=5)                            # nothing is measured twice
     assert not calls and plan == before
@@ -456,8 +456,7 @@ def test_products_are_measured_once_and_the_plan_is_followed(ops, monkeypatch):
     assert ops.route_linear(1, 768, 256, torch.bfloat16) == "skinny"            # the rule
     key = (1, 768, 256, False, torch.bfloat16)
     for seconds, choice in (([1.0, 0.95, 0.5, 0.96, 0.97], "resident256"), ([0.9, 0.95, 1.0, 0.96, 0.97], None)):
-        it = iter(seconds)
-        monkeypatch.setattr(ops, "_time_over", lambda *a: next(it))
+        monkeypatch.setattr(ops, "_time_ways", lambda runs, *a, seconds=seconds: dict(zip(runs, seconds)))
         plan.clear(); measured.clear()
         ops.tune_products([(ws[0], False, None)], max_rows=1)
         assert plan.get(key) == choice and measured[key] == choice
@@ -658,6 +657,35 @@ def test_prefill_attention_every_head_size(ops, ref, D, key_split, small_tiles, 
         ops.attention(q, a, kp, vp, step, 0, D ** -0.5, window)
         ref.attention(q, b, kp, vp, step, 0, D ** -0.5, window)
         torch.testing.assert_close(a.float(), b.float(), **tol(torch.bfloat16))
+
+
+def test_mixed_step_runs_its_two_attention_kernels_side_by_side(ops, ref, monkeypatch):
+    """A step of prompt portions beside decoded tokens: the decode kernel and the prefill kernel on two
+    streams give the bits they give one after the other, call after call (the second stream is joined
+    before anything reads the result), and what the plain reference gives."""
+    Hq, Hkv, D, P = 8, 2, 128, 16
+    segs = [(1, 700), (300, 40), (1, 5), (1, 1999), (70, 0), (1, 64), (2, 130)]
+    need = [-(-(a + b) // P) for a, b in segs]
+    perm = torch.randperm(sum(need) + 3, generator=torch.Generator().manual_seed(9)).tolist()
+    pages_of = [[perm.pop() for _ in range(k)] for k in need]
+    step = _step([s[0] for s in segs], [s[1] for s in segs], P, pages_of)
+    assert step.n_decode == 4 and step.n_prefill_tokens == 372
+    kp = rnd(sum(need) + 3, Hkv, P, D, dtype=torch.bfloat16, seed=61)
+    vp = rnd(sum(need) + 3, Hkv, P, D, dtype=torch.bfloat16, seed=62)
+    want = None
+    for it in range(6):
+        q = rnd(sum(s[0] for s in segs), Hq, D, dtype=torch.bfloat16, seed=70 + it)
+        outs = []
+        for overlap in (True, False):
+            monkeypatch.setattr(ops, "overlap_attention", overlap)
+            o = torch.zeros_like(q)
+            ops.attention(q, o, kp, vp, step, 0, D ** -0.5, 0)
+            outs.append(o * 1)                    # (read on the main stream, right after the call)
+        assert torch.equal(outs[0], outs[1]), f"call {it}"
+        want = torch.zeros_like(q)
+        ref.attention(q, want, kp, vp, step, 0, D ** -0.5, 0)
+        torch.testing.assert_close(outs[0].float(), want.float(), **tol(torch.bfloat16))
+    assert ops._side_stream is not None
 
 
 @pytest.mark.parametrize("merge", [0, 2, 4, 8])
