@@ -680,3 +680,80 @@ def test_layer_with_pages_and_state_and_a_second_position_axis_on_cpu_stand_in()
 def test_layer_with_pages_and_state_and_a_second_position_axis_on_gpu(use_graphs):
     runner = run_hybrid("cuda:0", None, use_graphs=use_graphs)
     assert bool(runner._graphs) == use_graphs
+
+
+# ------------------------------------------------------------------ a part that notes its products and forms them itself
+class PlainFeedForward:
+    """down(relu(up(x))). It names its first and last product (so that a kernel set may measure them) but its
+    forward has no ``sink`` parameter: it forms its last product itself, and no norm is finished inside it."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        return {"up": (params["intermediate_size"], params["hidden_size"]),
+                "down": (params["hidden_size"], params["intermediate_size"])}
+
+    @staticmethod
+    def random_init(params, role):
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.up = rt.product(rt.matrix(tensors["up"]))
+        self.down = rt.product(rt.matrix(tensors["down"]), residual=True)
+        self.first_product = (self.up, False)
+        self.last_product = self.down
+
+    def forward(self, x, step=None):
+        from return_amd.parts.runtime import ScaledRows
+        assert not isinstance(x, ScaledRows) or hasattr(self.rt.ops, "linear_add_norm")
+        return self.rt.ops.linear(self.rt.ops.linear(x, self.up).relu().contiguous(), self.down)
+
+
+register_part("feed_forward", "toy_plain_ff", PlainFeedForward)
+
+
+def test_a_part_without_a_sink_parameter_is_never_handed_one():
+    """PreNormBlock gives a part a sink for its last product only if the part's forward takes one: a part
+    that sets last_product and keeps the plain signature runs as it is, on a kernel set that would finish
+    norms inside products (the stand-in says it can, for up to 16 rows), in steps of one and of many rows."""
+    from return_amd.parts.block import takes_sink
+    from tests.torch_ops import TorchOps
+    cfg = ToyConfig.from_dict(dict(TOY, architectures=["ToyPlainFFForTests"]))
+    H = cfg.hidden_size
+    norm = lambda name: PartSpec("rms_norm", {"size": H, "eps": cfg.eps}, {"weight": name})
+    attn = PartSpec("attention", {"hidden_size": H, "num_heads": cfg.heads, "num_kv_heads": cfg.kv_heads,
+                                  "head_dim": cfg.head_dim, "scale": None, "window": None, "qk_norm_eps": None,
+                                  "position": None},
+                    {r: f"b.{r}" for r in ("q_proj", "k_proj", "v_proj", "o_proj")})
+    ff = PartSpec("toy_plain_ff", {"hidden_size": H, "intermediate_size": cfg.intermediate_size}, {"up": "b.up", "down": "b.down"})
+    spec = ModelSpec(
+        architecture=cfg.architecture, hidden_size=H, vocab_size=cfg.vocab_size, max_position=cfg.max_position_embeddings,
+        embedding=PartSpec("token_embedding", {"vocab_size": cfg.vocab_size, "hidden_size": H}, {"weight": "embed"}),
+        positions={}, blocks=[BlockSpec.pre_norm(attn, ff, norm("b.n1"), norm("b.n2"))],
+        schedule=[LayerCall(0, cache=0), LayerCall(0, cache=1)], final_norm=norm("final_norm"),
+        head=PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "hidden_size": H}, {"weight": "head"}))
+    register_architecture("ToyPlainFFForTests", ToyConfig, lambda c: spec)
+    weights = random_weights(spec, seed=3, std=0.08, norm_jitter=0.05, dtype="float32")
+    ec = EngineConfig(dtype="float32", page_size=4, max_token=256, max_reside=4, max_step_tokens=64, prefill_chunk=64,
+                      device="cpu", check_invariants=True)
+    runner = ModelRunner(config=cfg, weights=weights, engine_config=ec, ops=TorchOps())
+    block = runner.model.blocks[0]
+    assert takes_sink(block.mixer) and not takes_sink(block.feed_forward)
+    toks = tt.random_tokens(cfg.vocab_size, 30, seed=2)
+    from return_amd.engine import StepEntry
+    runner.add_request("whole")
+    whole = runner.step([StepEntry("whole", toks, list(range(30)))])
+    runner.add_request("cut")
+    rows = [runner.step([StepEntry("cut", toks[:9], list(range(9)))])]
+    rows += [runner.step([StepEntry("cut", [t], [0])]) for t in toks[9:]]          # single rows: norms inside products where they may be
+    torch.testing.assert_close(torch.cat(rows), whole, atol=2e-5, rtol=1e-4)
+
+
+def test_a_request_brings_a_column_value_for_its_prompt_tokens_at_most():
+    from return_amd.engine.scheduler import Request
+    r = Request("r", [1, 2, 3, 4], token_columns={"row": [0, 0, 1]})
+    assert r.columns_at(0, 4) == {"row": [0, 0, 1, 2]} and r.columns_at(3, 3) == {"row": [2, 3, 4]}
+    assert Request("s", [1, 2]).columns_at(0, 2) is None
+    for bad in ([], [0, 0, 0, 0, 0]):
+        with pytest.raises(ValueError, match="column"):
+            Request("t", [1, 2, 3, 4], token_columns={"row": bad})
