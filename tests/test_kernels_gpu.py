@@ -659,6 +659,29 @@ def test_prefill_attention_every_head_size(ops, ref, D, key_split, small_tiles, 
         torch.testing.assert_close(a.float(), b.float(), **tol(torch.bfloat16))
 
 
+def test_splits_of_the_decode_attention_follow_the_class_the_runner_names(ops):
+    """A decode step that names its class (the batch size and context bucket of the graph that serves or would
+    serve it) gets the class's splits, whatever its own numbers: the eager step of 12 requests of up to 301 tokens
+    and the captured step of 16 rows bound by 512 choose alike, and so sum in the same order. Without a class the
+    step's own numbers decide. Few waves: one pass of 64 keys each; the whole-round rule for merging inside the
+    workgroup follows the class too."""
+    def step(n, longest, rule=None, bound=False):
+        return types.SimpleNamespace(n_decode=n, max_decode_seq_len=longest, decode_rule=rule, decode_len_is_bound=bound)
+    n_q, n_kv, D = 32, 8, 128
+    eager = ops._decode_splits(step(12, 301, rule=(16, 512)), n_q, n_kv, D, 0)
+    graph = ops._decode_splits(step(16, 512, rule=(16, 512), bound=True), n_q, n_kv, D, 0)
+    assert eager[0] == graph[0] and eager[2] == graph[2] is False
+    assert graph[1] == (512 - 1) // graph[0] + 1 and eager[1] == (301 - 1) // eager[0] + 1
+    # one request over 2,048 keys: 8 kv heads x 33 chunks are few waves, a pass of 64 keys each
+    assert ops._decode_splits(step(1, 2049), n_q, n_kv, D, 0) == (64, 33, False)
+    assert ops._decode_splits(step(8, 2049), n_q, n_kv, D, 0)[0] == 128
+    # 32 requests x 8 kv heads are one whole round of the CUs (when the chip has 256): merged in the workgroup
+    if ops.cu_count == 256:
+        assert ops._decode_splits(step(32, 2049), n_q, n_kv, D, 0)[2] is True
+        assert ops._decode_splits(step(30, 2049, rule=(32, 4096)), n_q, n_kv, D, 0)[2] is True
+        assert ops._decode_splits(step(30, 2049), n_q, n_kv, D, 0)[2] is False
+
+
 def test_mixed_step_runs_its_two_attention_kernels_side_by_side(ops, ref, monkeypatch):
     """A step of prompt portions beside decoded tokens: the decode kernel and the prefill kernel on two
     streams give the bits they give one after the other, call after call (the second stream is joined
