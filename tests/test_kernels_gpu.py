@@ -36,7 +36,7 @@ DTYPES = [torch.float32, torch.bfloat16]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("V,H,T", [(331, 120, 7), (1000, 4096, 3)])
+@pytest.mark.parametrize("V,H,T", [(331, 120, 7), (1000, 4096, 3), (97, 100, 5), (500, 2560, 9), (64, 5120, 2)])
 def test_embed(ops, ref, dtype, V, H, T):
     table = rnd(V, H, dtype=dtype)
     ids = torch.randint(0, V, (T,), dtype=torch.int32, device=DEV)
