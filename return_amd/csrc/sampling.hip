@@ -97,10 +97,15 @@ __device__ __forceinline__ fixed_t block_sum_fixed(fixed_t v, fixed_t* wsum) {
 // A range of 2^32 keys takes three passes. wsum: CAND_WAVES words, sh_b, sh_above: one word each, all LDS.
 #define SEARCH_BITS 11
 #define SEARCH_BUCKETS (1 << SEARCH_BITS)
-// above (may be nullptr) is told measure{key > t}.
+// above (may be nullptr) is told measure{key > t}; at (may be nullptr) measure{key == t} where the last pass has
+// it (its run of the key range was the one key t), else FIXED_UNKNOWN (t is the lo it was given, whose tokens no
+// pass visits).
+#define FIXED_UNKNOWN (~0ull)
 template <typename Visit>
 __device__ uint32_t search_threshold(Visit visit, int tid, uint32_t lo, uint32_t hi, fixed_t limit, fixed_t* fx,
-                                     fixed_t* wsum, int* sh_b, fixed_t* sh_above, fixed_t* above = nullptr) {
+                                     fixed_t* wsum, int* sh_b, fixed_t* sh_above, fixed_t* above = nullptr,
+                                     fixed_t* at = nullptr) {
+    fixed_t at_t = FIXED_UNKNOWN;
     static_assert(SEARCH_BUCKETS == 2 * SAMPLE_THREADS, "a thread looks after two runs");
     const int wave = tid >> 6, lane = tid & 63;
     fixed_t above_hi = 0ull;
@@ -142,9 +147,11 @@ __device__ uint32_t search_threshold(Visit visit, int tid, uint32_t lo, uint32_t
         const uint32_t new_hi = end < (unsigned long long)hi ? (uint32_t)end : hi;
         lo = b == 0 ? lo : lo + ((uint32_t)b << sh);
         hi = new_hi;
+        if (lo == hi && b > 0) at_t = fx[b];           // the run was that one key: what was added into it is the key's
         __syncthreads();
     }
     if (above) *above = above_hi;
+    if (at) *at = at_t;
     return lo;
 }
 
@@ -153,12 +160,16 @@ __device__ uint32_t search_threshold(Visit visit, int tid, uint32_t lo, uint32_t
 // with index <= upto. One pass counts them; only if they are more than may stay, the index is searched.
 // (A function of its own, not inlined: it runs four times in the kernel, and inlined the kernel no longer
 // fits the 128 registers that a block of 1,024 threads leaves a lane.)
+// known: their number if the search has it already (then nothing is counted), else FIXED_UNKNOWN.
 template <typename Ties>
-__device__ __noinline__ int tie_cut(Ties ties, int tid, int V, unsigned long long stay, int upto, fixed_t* fx, fixed_t* wsum,
-                       int* sh_b, fixed_t* sh_above) {
-    fixed_t mine = 0ull;
-    ties([&](int) { mine += 1ull; });
-    const fixed_t n = block_sum_fixed(mine, wsum);
+__device__ __noinline__ int tie_cut(Ties ties, int tid, int V, unsigned long long stay, int upto, fixed_t known,
+                       fixed_t* fx, fixed_t* wsum, int* sh_b, fixed_t* sh_above) {
+    fixed_t n = known;
+    if (known == FIXED_UNKNOWN) {
+        fixed_t mine = 0ull;
+        ties([&](int) { mine += 1ull; });
+        n = block_sum_fixed(mine, wsum);
+    }
     if (stay >= n) return upto;
     if (stay == 0ull) return -1;
     // the stay-th tie from the front: the smallest t with at most stay - 1 ties at keys V - 1 - index above it
@@ -386,17 +397,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                 };
                 // top-k: the k-th largest is on the list; below cut_key - 1 nothing of it lies
                 if (want_k) {
-                    fixed_t above = 0ull;
+                    fixed_t above = 0ull, at = FIXED_UNKNOWN;
                     keep_key = search_threshold(
                         [&](uint32_t lo, uint32_t hi, auto add) {
 #pragma unroll
                             for (int e = 0; e < CAND_OWN; ++e)
                                 if (key[e] > lo && key[e] <= hi) add(key[e], 1ull << 40);
                         },
-                        tid, cut_key - 1u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above, &above);
+                        tid, cut_key - 1u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above, &above, &at);
                     // of the tokens that tie with the k-th value, as many stay as make k with those above them
                     tie_limit = tie_cut(ties_at(keep_key, 0x7fffffff), tid, V, (unsigned long long)k - (above >> 40),
-                                        0x7fffffff, fx, wsum, &sh_b, &sh_above);
+                                        0x7fffffff, at == FIXED_UNKNOWN ? at : at >> 40, fx, wsum, &sh_b, &sh_above);
                 }
                 if (want_p) {
                     fixed_t zc = 0ull;
@@ -409,7 +420,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                     if (want_k || zc > limit) {
                         const uint32_t k_key = keep_key;     // what top-k left: the search goes over that
                         const int k_limit = tie_limit;
-                        fixed_t above = 0ull;
+                        fixed_t above = 0ull, at = FIXED_UNKNOWN;
                         keep_key = search_threshold(
                             [&](uint32_t lo, uint32_t hi, auto add) {
 #pragma unroll
@@ -417,13 +428,15 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                                     if (idx[e] >= 0 && key[e] > lo && key[e] <= hi &&
                                         (key[e] > k_key || idx[e] <= k_limit)) add(key[e], to_fixed(weight[e]));
                             },
-                            tid, want_k ? k_key : cut_key - 1u, top_key, limit, fx, wsum, &sh_b, &sh_above, &above);
+                            tid, want_k ? k_key : cut_key - 1u, top_key, limit, fx, wsum, &sh_b, &sh_above, &above, &at);
                         // of the tokens that tie with the boundary value, the i-th in vocabulary order stays while
                         // what lies before it, the mass above them and i of their own, is at most top_p of the whole
                         const fixed_t each = to_fixed(__expf((key_value(keep_key) - gmax) * inv_t));
                         const unsigned long long stay = each ? (limit - above) / each + 1ull : ~0ull;
                         const int upto = keep_key == k_key ? k_limit : 0x7fffffff;
-                        tie_limit = tie_cut(ties_at(keep_key, upto), tid, V, stay, upto, fx, wsum, &sh_b, &sh_above);
+                        // (a boundary above top-k's: every token of that value was in the search, their mass is their number)
+                        const fixed_t known = (at != FIXED_UNKNOWN && each && (!want_k || keep_key != k_key)) ? at / each : FIXED_UNKNOWN;
+                        tie_limit = tie_cut(ties_at(keep_key, upto), tid, V, stay, upto, known, fx, wsum, &sh_b, &sh_above);
                     } else {
                         listed = false;
                     }
@@ -492,7 +505,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         // ---- over the whole row. top-k: the key of the k-th largest value is the smallest key with at most
         // k - 1 tokens above it
         if (want_k) {
-            fixed_t above = 0ull;
+            fixed_t above = 0ull, at = FIXED_UNKNOWN;
             keep_key = search_threshold(
                 [&](uint32_t lo, uint32_t hi, auto add) {
                     for_each_logit(x, V, tid, [&](int, float v) {
@@ -500,9 +513,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                         if (key > lo && key <= hi) add(key, 1ull << 40);
                     });
                 },
-                tid, 0u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above, &above);
+                tid, 0u, top_key, (fixed_t)(k - 1) << 40, fx, wsum, &sh_b, &sh_above, &above, &at);
             tie_limit = tie_cut(ties_at(keep_key, 0x7fffffff), tid, V, (unsigned long long)k - (above >> 40),
-                                0x7fffffff, fx, wsum, &sh_b, &sh_above);
+                                0x7fffffff, at == FIXED_UNKNOWN ? at : at >> 40, fx, wsum, &sh_b, &sh_above);
         }
         // top-p: the smallest key with at most p of the kept mass above it
         if (want_p) {
@@ -514,7 +527,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             const fixed_t limit = (fixed_t)((double)p * (double)z);
             const uint32_t k_key = keep_key;             // what top-k left: the search goes over that
             const int k_limit = tie_limit;
-            fixed_t above = 0ull;
+            fixed_t above = 0ull, at = FIXED_UNKNOWN;
             keep_key = search_threshold(
                 [&](uint32_t lo, uint32_t hi, auto add) {
                     for_each_logit(x, V, tid, [&](int i, float v) {
@@ -523,11 +536,12 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                             add(key, to_fixed(__expf((v - gmax) * inv_t)));
                     });
                 },
-                tid, k_key, top_key, limit, fx, wsum, &sh_b, &sh_above, &above);
+                tid, k_key, top_key, limit, fx, wsum, &sh_b, &sh_above, &above, &at);
             const fixed_t each = to_fixed(__expf((key_value(keep_key) - gmax) * inv_t));
             const unsigned long long stay = each ? (limit - above) / each + 1ull : ~0ull;
             const int upto = keep_key == k_key ? k_limit : 0x7fffffff;
-            tie_limit = tie_cut(ties_at(keep_key, upto), tid, V, stay, upto, fx, wsum, &sh_b, &sh_above);
+            const fixed_t known = (at != FIXED_UNKNOWN && each && (!want_k || keep_key != k_key)) ? at / each : FIXED_UNKNOWN;
+            tie_limit = tie_cut(ties_at(keep_key, upto), tid, V, stay, upto, known, fx, wsum, &sh_b, &sh_above);
         }
     }
 
